@@ -1,0 +1,121 @@
+/*
+ * hiprwkv -- C ABI of the MI355X (gfx950) WKV recurrence library.
+ *
+ * Every entry point only enqueues work on the caller's HIP stream: it does not
+ * allocate, free or synchronise, so it can be called from an XLA custom-call
+ * handler thread.  All pointers are device pointers.  Entry points return
+ * HIPRWKV_OK or a negative HIPRWKV_E* code; hiprwkv_last_error() then returns a
+ * thread-local message.
+ *
+ * Operand order follows the reference's jax.ffi targets, whose native
+ * implementation (package `jaxrwkvkernel`, CUDA only) is not part of the
+ * reference tree; each declaration cites the Python call site it replaces.
+ *
+ * Shapes: B sequences (the reference's vmap axis), T tokens, H heads, N head size.
+ *   WKV7/WKV6 token tensors  (B,T,H,N) row-major, io_dtype
+ *   WKV7 state               (B,H,N,N) state_dtype, s[b,h,i,j]: value row i, key column j
+ *   WKV6 state               (B,H,N,N) state_dtype, s[b,h,i,j]: key row i, value column j
+ *   WKV4 token tensors       (B,T,C), state (B,3,C) = (aa,bb,pp)
+ *   length                   (B,) uint32, may be NULL (= T)
+ *   new_starts               (B,T) one byte per token (0/1), may be NULL (= none)
+ * The recurrence always runs in fp32 whatever the io/state dtypes are.
+ */
+#ifndef HIPRWKV_H_
+#define HIPRWKV_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HIPRWKV_OK 0
+#define HIPRWKV_EINVAL (-1)   /* bad argument (shape, dtype, NULL pointer) */
+#define HIPRWKV_ELAUNCH (-2)  /* hipLaunchKernel reported an error */
+#define HIPRWKV_ENOSPACE (-3) /* workspace too small */
+
+#define HIPRWKV_F32 0
+#define HIPRWKV_BF16 1
+
+/* flags */
+/* Reproduce AssociativeScanRWKV where it differs from the sequential loop:
+ * WKV7 y[t] = 0 when new_starts[t+1] (rwkv7.py:331-333,344); returned state is the
+ * one entering position `length` (rwkv7.py:345, rwkv6.py:301, rwkv4.py:300). */
+#define HIPRWKV_COMPAT_ASSOC 1u
+/* Force the sequential fp32 VALU kernel even where a chunked MFMA kernel exists. */
+#define HIPRWKV_FORCE_SEQ 2u
+
+typedef void* hiprwkv_stream; /* a hipStream_t */
+
+const char* hiprwkv_last_error(void);
+int hiprwkv_version(void);
+
+/* ---- WKV7 ------------------------------------------------------------------
+ * Replaces ffi target "wkv7-fwd-{fp32,bf16}": operands w,r,k,v,a,b,s,length,new_starts
+ * -> out, s_restore, sa_restore, new_s  (rwkv7.py:372-375).  `w` is the raw decay
+ * argument; the op applies exp(-exp(w)) (rwkv7.py:201).  `sa` (B,T,H,N) fp32 is
+ * the residual S_{t-1} a_t kept for the backward pass (the reference's sa_restore);
+ * pass NULL for inference.  No state checkpoints (s_restore) are needed. */
+int hiprwkv_wkv7_fwd(hiprwkv_stream stream, int io_dtype, int state_dtype,
+                     int64_t B, int64_t T, int64_t H, int64_t N,
+                     const void* w, const void* r, const void* k, const void* v,
+                     const void* a, const void* b, const void* s,
+                     const uint32_t* length, const uint8_t* new_starts,
+                     void* out, float* sa, void* new_s, unsigned flags);
+
+/* Bytes of scratch hiprwkv_wkv7_bwd needs for this shape. */
+size_t hiprwkv_wkv7_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t N);
+
+/* Replaces ffi target "wkv7-bwd-{fp32,bf16}": operands w,r,k,v,a,b,s,length,new_starts,
+ * gy,s_restore,sa_restore,gs_out -> gw,gr,gk,gv,ga,gb,gs  (rwkv7.py:406-408).
+ * Unlike the reference's native op it honours new_starts, takes the cotangent of the
+ * returned state (gs_out, may be NULL = 0) and returns the one of the input state. */
+int hiprwkv_wkv7_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype,
+                     int64_t B, int64_t T, int64_t H, int64_t N,
+                     const void* w, const void* r, const void* k, const void* v,
+                     const void* a, const void* b, const void* s,
+                     const uint32_t* length, const uint8_t* new_starts,
+                     const void* gy, const float* sa, const void* gs_out,
+                     void* gw, void* gr, void* gk, void* gv, void* ga, void* gb, void* gs,
+                     void* workspace, size_t workspace_bytes, unsigned flags);
+
+/* ---- WKV6 ------------------------------------------------------------------
+ * The reference has no native WKV6 op (README.md:93-99); the operand order follows
+ * inner_loop(r,k,v,w,time_first,s,length,new_starts) (rwkv6.py:175).  `w` is the log
+ * decay -exp(raw) (rwkv6.py:217-218), `u` = time_faaaa (H,N) io_dtype. */
+int hiprwkv_wkv6_fwd(hiprwkv_stream stream, int io_dtype, int state_dtype,
+                     int64_t B, int64_t T, int64_t H, int64_t N,
+                     const void* r, const void* k, const void* v, const void* w,
+                     const void* u, const void* s,
+                     const uint32_t* length, const uint8_t* new_starts,
+                     void* out, void* new_s, unsigned flags);
+
+size_t hiprwkv_wkv6_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t N);
+
+/* Cotangents of wkv6_fwd: gr,gk,gv,gw (B,T,H,N) io_dtype; gu (B,H,N) fp32, to be summed
+ * over B by the caller (as the reference does for the WKV4 parameters, rwkv4.py:351);
+ * gs (B,H,N,N) state_dtype. */
+int hiprwkv_wkv6_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype,
+                     int64_t B, int64_t T, int64_t H, int64_t N,
+                     const void* r, const void* k, const void* v, const void* w,
+                     const void* u, const void* s,
+                     const uint32_t* length, const uint8_t* new_starts,
+                     const void* gy, const void* gs_out,
+                     void* gr, void* gk, void* gv, void* gw, float* gu, void* gs,
+                     void* workspace, size_t workspace_bytes, unsigned flags);
+
+/* ---- WKV4 ------------------------------------------------------------------
+ * Replaces ffi target "wkv4-fwd-{fp32,bf16}": operands w,time_first,k,v,s,length,new_starts
+ * -> new_s, out  (rwkv4.py:320-321).  `w` = -exp(time_decay) (rwkv4.py:312) and `u` are (C,)
+ * io_dtype; the receptance is applied by the caller (rwkv4.py:406). */
+int hiprwkv_wkv4_fwd(hiprwkv_stream stream, int io_dtype,
+                     int64_t B, int64_t T, int64_t C,
+                     const void* w, const void* u, const void* k, const void* v, const void* s,
+                     const uint32_t* length, const uint8_t* new_starts,
+                     void* new_s, void* out, unsigned flags);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HIPRWKV_H_ */

@@ -1,0 +1,59 @@
+"""ctypes binding of ``libhiprwkv.so`` (the C ABI declared in ``include/hiprwkv.h``).
+
+There is no fallback: if the library has not been built, or a call fails, an exception is raised.
+"""
+import ctypes
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libhiprwkv.so")
+
+F32, BF16 = 0, 1
+COMPAT_ASSOC = 1
+FORCE_SEQ = 2
+
+_vp, _i64, _int, _u32, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_uint, ctypes.c_size_t
+
+# name -> (restype, argtypes); mirrors include/hiprwkv.h declaration by declaration
+SIGNATURES = {
+    "hiprwkv_last_error": (ctypes.c_char_p, []),
+    "hiprwkv_version": (_int, []),
+    "hiprwkv_wkv7_fwd": (_int, [_vp, _int, _int, _i64, _i64, _i64, _i64] + [_vp] * 7 + [_vp, _vp] + [_vp, _vp, _vp, _u32]),
+    "hiprwkv_wkv7_bwd_workspace_bytes": (_sz, [_i64] * 4),
+    "hiprwkv_wkv7_bwd": (_int, [_vp, _int, _int, _i64, _i64, _i64, _i64] + [_vp] * 7 + [_vp, _vp] + [_vp] * 3
+                         + [_vp] * 7 + [_vp, _sz, _u32]),
+    "hiprwkv_wkv6_fwd": (_int, [_vp, _int, _int, _i64, _i64, _i64, _i64] + [_vp] * 6 + [_vp, _vp] + [_vp, _vp, _u32]),
+    "hiprwkv_wkv6_bwd_workspace_bytes": (_sz, [_i64] * 4),
+    "hiprwkv_wkv6_bwd": (_int, [_vp, _int, _int, _i64, _i64, _i64, _i64] + [_vp] * 6 + [_vp, _vp] + [_vp, _vp]
+                         + [_vp] * 6 + [_vp, _sz, _u32]),
+    "hiprwkv_wkv4_fwd": (_int, [_vp, _int, _i64, _i64, _i64] + [_vp] * 5 + [_vp, _vp] + [_vp, _vp, _u32]),
+}
+
+_lib = None
+
+
+class HipRwkvError(RuntimeError):
+    pass
+
+
+def load():
+    """Loads the library once and types every entry point; raises if it is missing."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise HipRwkvError(
+            f"{LIB_PATH} is missing: build it with `python -m jaxrwkv_amd.build` (there is no CPU fallback)")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(rc, what):
+    if rc != 0:
+        msg = load().hiprwkv_last_error().decode()
+        raise HipRwkvError(f"{what} failed with code {rc}: {msg}")

@@ -1,0 +1,189 @@
+// C ABI of libhiprwkv: argument checks, workspace carving, kernel selection.  Declarations: include/hiprwkv.h
+#include "../../include/hiprwkv.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include "wkv_args.h"
+
+using namespace hiprwkv;
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+bool dtype_ok(int d) { return d == HIPRWKV_F32 || d == HIPRWKV_BF16; }
+
+size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+int check_matrix_shape(const char* op, int io_dtype, int state_dtype, int64_t B, int64_t T, int64_t H, int64_t N) {
+  if (!dtype_ok(io_dtype) || !dtype_ok(state_dtype)) return fail(HIPRWKV_EINVAL, "%s: dtype must be HIPRWKV_F32 or HIPRWKV_BF16", op);
+  if (N != 64) return fail(HIPRWKV_EINVAL, "%s: head size N=%lld not supported (kernels are built for N=64)", op, (long long)N);
+  if (B <= 0 || T <= 0 || H <= 0) return fail(HIPRWKV_EINVAL, "%s: B,T,H must be positive (got %lld,%lld,%lld)", op, (long long)B, (long long)T, (long long)H);
+  if (B * H > 0x7fffffffLL) return fail(HIPRWKV_EINVAL, "%s: B*H exceeds the grid limit", op);
+  return HIPRWKV_OK;
+}
+
+bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+}  // namespace
+
+extern "C" {
+
+const char* hiprwkv_last_error(void) { return g_err; }
+int hiprwkv_version(void) { return 100; }
+
+int hiprwkv_wkv7_fwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64_t B, int64_t T, int64_t H, int64_t N,
+                     const void* w, const void* r, const void* k, const void* v, const void* a, const void* b,
+                     const void* s, const uint32_t* length, const uint8_t* new_starts, void* out, float* sa,
+                     void* new_s, unsigned flags) {
+  int rc = check_matrix_shape("wkv7_fwd", io_dtype, state_dtype, B, T, H, N);
+  if (rc) return rc;
+  const void* req[] = {w, r, k, v, a, b, s, out, new_s};
+  for (const void* p : req) {
+    if (p == nullptr) return fail(HIPRWKV_EINVAL, "wkv7_fwd: null tensor pointer");
+    if (!aligned16(p)) return fail(HIPRWKV_EINVAL, "wkv7_fwd: tensor pointers must be 16-byte aligned");
+  }
+  if (sa && !aligned16(sa)) return fail(HIPRWKV_EINVAL, "wkv7_fwd: sa must be 16-byte aligned");
+  Wkv7Args A;
+  memset(&A, 0, sizeof(A));
+  A.B = B; A.T = T; A.H = H;
+  A.w = w; A.r = r; A.k = k; A.v = v; A.a = a; A.b = b; A.s = s;
+  A.length = length; A.ns = new_starts;
+  A.out = out; A.sa = sa; A.new_s = new_s;
+  A.io_f32 = io_dtype == HIPRWKV_F32; A.st_f32 = state_dtype == HIPRWKV_F32;
+  A.flags = flags;
+  hipError_t e = launch_wkv7_seq_fwd(A, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "wkv7_fwd: %s", hipGetErrorString(e));
+  return HIPRWKV_OK;
+}
+
+size_t hiprwkv_wkv7_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t N) {
+  return 3 * align256((size_t)B * T * H * N * sizeof(float));
+}
+
+int hiprwkv_wkv7_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64_t B, int64_t T, int64_t H, int64_t N,
+                     const void* w, const void* r, const void* k, const void* v, const void* a, const void* b,
+                     const void* s, const uint32_t* length, const uint8_t* new_starts, const void* gy, const float* sa,
+                     const void* gs_out, void* gw, void* gr, void* gk, void* gv, void* ga, void* gb, void* gs,
+                     void* workspace, size_t workspace_bytes, unsigned flags) {
+  int rc = check_matrix_shape("wkv7_bwd", io_dtype, state_dtype, B, T, H, N);
+  if (rc) return rc;
+  const void* req[] = {w, r, k, v, a, b, s, gy, sa, gw, gr, gk, gv, ga, gb, gs, workspace};
+  for (const void* p : req) {
+    if (p == nullptr) return fail(HIPRWKV_EINVAL, "wkv7_bwd: null tensor pointer");
+    if (!aligned16(p)) return fail(HIPRWKV_EINVAL, "wkv7_bwd: tensor pointers must be 16-byte aligned");
+  }
+  const size_t need = hiprwkv_wkv7_bwd_workspace_bytes(B, T, H, N);
+  if (workspace_bytes < need)
+    return fail(HIPRWKV_ENOSPACE, "wkv7_bwd: workspace has %zu bytes, %zu needed", workspace_bytes, need);
+  Wkv7Args A;
+  memset(&A, 0, sizeof(A));
+  A.B = B; A.T = T; A.H = H;
+  A.w = w; A.r = r; A.k = k; A.v = v; A.a = a; A.b = b; A.s = s;
+  A.length = length; A.ns = new_starts;
+  A.io_f32 = io_dtype == HIPRWKV_F32; A.st_f32 = state_dtype == HIPRWKV_F32;
+  A.flags = flags;
+  A.gy = gy; A.sa_in = sa; A.gs_out = gs_out;
+  A.gw = gw; A.gr = gr; A.gk = gk; A.gv = gv; A.ga = ga; A.gb = gb; A.gs = gs;
+  const size_t one = need / 3;
+  char* ws = static_cast<char*>(workspace);
+  A.dsa = reinterpret_cast<float*>(ws);
+  A.e2 = reinterpret_cast<float*>(ws + one);
+  A.e3 = reinterpret_cast<float*>(ws + 2 * one);
+  hipError_t e = launch_wkv7_seq_bwd(A, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "wkv7_bwd: %s", hipGetErrorString(e));
+  return HIPRWKV_OK;
+}
+
+int hiprwkv_wkv6_fwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64_t B, int64_t T, int64_t H, int64_t N,
+                     const void* r, const void* k, const void* v, const void* w, const void* u, const void* s,
+                     const uint32_t* length, const uint8_t* new_starts, void* out, void* new_s, unsigned flags) {
+  int rc = check_matrix_shape("wkv6_fwd", io_dtype, state_dtype, B, T, H, N);
+  if (rc) return rc;
+  const void* req[] = {r, k, v, w, u, s, out, new_s};
+  for (const void* p : req) {
+    if (p == nullptr) return fail(HIPRWKV_EINVAL, "wkv6_fwd: null tensor pointer");
+    if (!aligned16(p)) return fail(HIPRWKV_EINVAL, "wkv6_fwd: tensor pointers must be 16-byte aligned");
+  }
+  Wkv6Args A;
+  memset(&A, 0, sizeof(A));
+  A.B = B; A.T = T; A.H = H;
+  A.r = r; A.k = k; A.v = v; A.w = w; A.u = u; A.s = s;
+  A.length = length; A.ns = new_starts;
+  A.out = out; A.new_s = new_s;
+  A.io_f32 = io_dtype == HIPRWKV_F32; A.st_f32 = state_dtype == HIPRWKV_F32;
+  A.flags = flags;
+  hipError_t e = launch_wkv6_seq_fwd(A, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "wkv6_fwd: %s", hipGetErrorString(e));
+  return HIPRWKV_OK;
+}
+
+size_t hiprwkv_wkv6_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t N) {
+  return align256((size_t)B * T * H * N * sizeof(float)) + align256((size_t)B * H * N * sizeof(float));
+}
+
+int hiprwkv_wkv6_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64_t B, int64_t T, int64_t H, int64_t N,
+                     const void* r, const void* k, const void* v, const void* w, const void* u, const void* s,
+                     const uint32_t* length, const uint8_t* new_starts, const void* gy, const void* gs_out, void* gr,
+                     void* gk, void* gv, void* gw, float* gu, void* gs, void* workspace, size_t workspace_bytes,
+                     unsigned flags) {
+  int rc = check_matrix_shape("wkv6_bwd", io_dtype, state_dtype, B, T, H, N);
+  if (rc) return rc;
+  const void* req[] = {r, k, v, w, u, s, gy, gr, gk, gv, gw, gu, gs, workspace};
+  for (const void* p : req) {
+    if (p == nullptr) return fail(HIPRWKV_EINVAL, "wkv6_bwd: null tensor pointer");
+    if (!aligned16(p)) return fail(HIPRWKV_EINVAL, "wkv6_bwd: tensor pointers must be 16-byte aligned");
+  }
+  const size_t need = hiprwkv_wkv6_bwd_workspace_bytes(B, T, H, N);
+  if (workspace_bytes < need)
+    return fail(HIPRWKV_ENOSPACE, "wkv6_bwd: workspace has %zu bytes, %zu needed", workspace_bytes, need);
+  Wkv6Args A;
+  memset(&A, 0, sizeof(A));
+  A.B = B; A.T = T; A.H = H;
+  A.r = r; A.k = k; A.v = v; A.w = w; A.u = u; A.s = s;
+  A.length = length; A.ns = new_starts;
+  A.io_f32 = io_dtype == HIPRWKV_F32; A.st_f32 = state_dtype == HIPRWKV_F32;
+  A.flags = flags;
+  A.gy = gy; A.gs_out = gs_out;
+  A.gr = gr; A.gk = gk; A.gv = gv; A.gw = gw; A.gu = gu; A.gs = gs;
+  char* ws = static_cast<char*>(workspace);
+  A.er = reinterpret_cast<float*>(ws);
+  A.eI = reinterpret_cast<float*>(ws + align256((size_t)B * T * H * N * sizeof(float)));
+  hipError_t e = launch_wkv6_seq_bwd(A, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "wkv6_bwd: %s", hipGetErrorString(e));
+  return HIPRWKV_OK;
+}
+
+int hiprwkv_wkv4_fwd(hiprwkv_stream stream, int io_dtype, int64_t B, int64_t T, int64_t C, const void* w,
+                     const void* u, const void* k, const void* v, const void* s, const uint32_t* length,
+                     const uint8_t* new_starts, void* new_s, void* out, unsigned flags) {
+  if (!dtype_ok(io_dtype)) return fail(HIPRWKV_EINVAL, "wkv4_fwd: dtype must be HIPRWKV_F32 or HIPRWKV_BF16");
+  if (B <= 0 || T <= 0 || C <= 0) return fail(HIPRWKV_EINVAL, "wkv4_fwd: B,T,C must be positive");
+  if (B * ((C + 63) / 64) > 0x7fffffffLL) return fail(HIPRWKV_EINVAL, "wkv4_fwd: B*C exceeds the grid limit");
+  const void* req[] = {w, u, k, v, s, new_s, out};
+  for (const void* p : req)
+    if (p == nullptr) return fail(HIPRWKV_EINVAL, "wkv4_fwd: null tensor pointer");
+  Wkv4Args A;
+  memset(&A, 0, sizeof(A));
+  A.B = B; A.T = T; A.C = C;
+  A.w = w; A.u = u; A.k = k; A.v = v; A.s = s;
+  A.length = length; A.ns = new_starts;
+  A.new_s = new_s; A.out = out;
+  A.io_f32 = io_dtype == HIPRWKV_F32;
+  A.flags = flags;
+  hipError_t e = launch_wkv4_fwd(A, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "wkv4_fwd: %s", hipGetErrorString(e));
+  return HIPRWKV_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,61 @@
+// Plain argument blocks passed by value to the kernels, and the launcher prototypes the C ABI calls.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace hiprwkv {
+
+struct Wkv7Args {
+  int64_t B, T, H;
+  const void *w, *r, *k, *v, *a, *b, *s;
+  const uint32_t* length;
+  const uint8_t* ns;
+  void* out;
+  float* sa;      // forward residual (may be null)
+  void* new_s;
+  int io_f32, st_f32;
+  unsigned flags;
+  // backward only
+  const void* gy;
+  const float* sa_in;
+  const void* gs_out;
+  void *gw, *gr, *gk, *gv, *ga, *gb, *gs;
+  float *dsa, *e2, *e3;  // workspace, (B,T,H,64) fp32 each
+};
+
+struct Wkv6Args {
+  int64_t B, T, H;
+  const void *r, *k, *v, *w, *u, *s;
+  const uint32_t* length;
+  const uint8_t* ns;
+  void* out;
+  void* new_s;
+  int io_f32, st_f32;
+  unsigned flags;
+  // backward only
+  const void* gy;
+  const void* gs_out;
+  void *gr, *gk, *gv, *gw, *gs;
+  float* gu;   // (B,H,64)
+  float* er;   // workspace (B,T,H,64): r . (S' dy)
+  float* eI;   // workspace (B,H,64): rowsum(dS_out * S_{length-1})
+};
+
+struct Wkv4Args {
+  int64_t B, T, C;
+  const void *w, *u, *k, *v, *s;
+  const uint32_t* length;
+  const uint8_t* ns;
+  void* new_s;
+  void* out;
+  int io_f32;
+  unsigned flags;
+};
+
+hipError_t launch_wkv7_seq_fwd(const Wkv7Args& A, hipStream_t stream);
+hipError_t launch_wkv7_seq_bwd(const Wkv7Args& A, hipStream_t stream);
+hipError_t launch_wkv6_seq_fwd(const Wkv6Args& A, hipStream_t stream);
+hipError_t launch_wkv6_seq_bwd(const Wkv6Args& A, hipStream_t stream);
+hipError_t launch_wkv4_fwd(const Wkv4Args& A, hipStream_t stream);
+
+}  // namespace hiprwkv

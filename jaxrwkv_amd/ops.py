@@ -1,0 +1,200 @@
+"""Host-side operators over device tensors: thin, allocation + pointer plumbing around the C ABI.
+
+Tensors are ``torch`` CUDA tensors (torch is used for device memory and streams only).  Every operator takes a
+leading batch axis ``B`` -- what the reference gets from ``jax.vmap`` (rwkv7.py:419-431) -- and enqueues on the
+current stream.  ``compat=True`` (default) reproduces ``AssociativeScanRWKV``; ``compat=False`` the sequential
+``BaseRWKV``/``ScanRWKV`` conventions (they differ only in y[t] when new_starts[t+1], and in the returned state
+when new_starts[length]).
+"""
+import torch
+
+from . import _lib
+
+_DT = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16}
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _p(t):
+    return None if t is None else t.data_ptr()
+
+
+def _dev(x, dtype=None):
+    if not x.is_cuda:
+        raise _lib.HipRwkvError("hiprwkv operators need CUDA (ROCm) tensors; there is no CPU path")
+    if dtype is not None and x.dtype != dtype:
+        x = x.to(dtype)
+    return x.contiguous()
+
+
+def _length_ns(length, new_starts, B, T, device):
+    if length is not None:
+        length = torch.as_tensor(length, device=device).to(torch.int32).reshape(-1)
+        if length.numel() == 1 and B > 1:
+            length = length.expand(B)
+        length = length.clamp(min=0).contiguous()
+        assert length.numel() == B
+    if new_starts is not None:
+        new_starts = torch.as_tensor(new_starts, device=device).to(torch.bool)
+        if new_starts.dim() == 1:
+            new_starts = new_starts[None].expand(B, T)
+        new_starts = new_starts.contiguous()
+        assert new_starts.shape == (B, T)
+    return length, new_starts
+
+
+def _flags(compat):
+    return _lib.COMPAT_ASSOC if compat else 0
+
+
+# ----------------------------------------------------------------------------- WKV7
+def wkv7_fwd(r, w, k, v, a, b, s, length=None, new_starts=None, compat=True, want_sa=False):
+    """r,w,k,v,a,b (B,T,H,N) fp32|bf16; s (B,H,N,N) fp32|bf16.  Returns (new_s, y, sa|None)."""
+    lib = _lib.load()
+    io = r.dtype
+    r, w, k, v, a, b = (_dev(x, io) for x in (r, w, k, v, a, b))
+    s = _dev(s)
+    B, T, H, N = r.shape
+    assert s.shape == (B, H, N, N), (s.shape, r.shape)
+    length, new_starts = _length_ns(length, new_starts, B, T, r.device)
+    y = torch.empty_like(r)
+    new_s = torch.empty_like(s)
+    sa = torch.empty((B, T, H, N), dtype=torch.float32, device=r.device) if want_sa else None
+    rc = lib.hiprwkv_wkv7_fwd(_stream(), _DT[io], _DT[s.dtype], B, T, H, N, _p(w), _p(r), _p(k), _p(v), _p(a), _p(b),
+                              _p(s), _p(length), _p(new_starts), _p(y), _p(sa), _p(new_s), _flags(compat))
+    _lib.check(rc, "hiprwkv_wkv7_fwd")
+    return new_s, y, sa
+
+
+def wkv7_bwd(r, w, k, v, a, b, s, length, new_starts, gy, sa, gs_out=None, compat=True):
+    """Cotangents (gr, gw, gk, gv, ga, gb, gs) of ``wkv7_fwd`` for cotangents gy of y and gs_out of new_s."""
+    lib = _lib.load()
+    io = r.dtype
+    r, w, k, v, a, b, gy = (_dev(x, io) for x in (r, w, k, v, a, b, gy))
+    s = _dev(s)
+    sa = _dev(sa, torch.float32)
+    gs_out = None if gs_out is None else _dev(gs_out, s.dtype)
+    B, T, H, N = r.shape
+    length, new_starts = _length_ns(length, new_starts, B, T, r.device)
+    gw, gr, gk, gv, ga, gb = (torch.empty_like(r) for _ in range(6))
+    gs = torch.empty_like(s)
+    nbytes = lib.hiprwkv_wkv7_bwd_workspace_bytes(B, T, H, N)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=r.device)
+    rc = lib.hiprwkv_wkv7_bwd(_stream(), _DT[io], _DT[s.dtype], B, T, H, N, _p(w), _p(r), _p(k), _p(v), _p(a), _p(b),
+                              _p(s), _p(length), _p(new_starts), _p(gy), _p(sa), _p(gs_out),
+                              _p(gw), _p(gr), _p(gk), _p(gv), _p(ga), _p(gb), _p(gs), _p(ws), nbytes, _flags(compat))
+    _lib.check(rc, "hiprwkv_wkv7_bwd")
+    return gr, gw, gk, gv, ga, gb, gs
+
+
+class _Wkv7(torch.autograd.Function):
+    """custom VJP, the counterpart of ``wkv7_cuda`` (rwkv7.py:442-446)."""
+
+    @staticmethod
+    def forward(ctx, r, w, k, v, a, b, s, length, new_starts, compat):
+        need = any(x.requires_grad for x in (r, w, k, v, a, b, s))
+        new_s, y, sa = wkv7_fwd(r, w, k, v, a, b, s, length, new_starts, compat, want_sa=need)
+        ctx.compat = compat
+        ctx.save_for_backward(r, w, k, v, a, b, s, length, new_starts, sa)
+        return new_s, y
+
+    @staticmethod
+    def backward(ctx, gs_out, gy):
+        r, w, k, v, a, b, s, length, new_starts, sa = ctx.saved_tensors
+        if gy is None:
+            gy = torch.zeros_like(r)
+        gr, gw, gk, gv, ga, gb, gs = wkv7_bwd(r, w, k, v, a, b, s, length, new_starts, gy, sa, gs_out, ctx.compat)
+        return gr, gw, gk, gv, ga, gb, gs, None, None, None
+
+
+def wkv7(r, w, k, v, a, b, s, length=None, new_starts=None, compat=True):
+    """Differentiable WKV7: returns (new_s, y)."""
+    B, T = r.shape[:2]
+    length, new_starts = _length_ns(length, new_starts, B, T, r.device)
+    return _Wkv7.apply(r, w, k, v, a, b, s, length, new_starts, compat)
+
+
+# ----------------------------------------------------------------------------- WKV6
+def wkv6_fwd(r, k, v, w, u, s, length=None, new_starts=None, compat=True):
+    """r,k,v,w (B,T,H,N); u (H,N); s (B,H,N,N) [key, value].  Returns (new_s, y)."""
+    lib = _lib.load()
+    io = r.dtype
+    B, T, H, N = r.shape
+    r, k, v = (_dev(x, io) for x in (r, k, v))
+    w = _dev(w.reshape(B, T, H, N), io)
+    u = _dev(u.reshape(H, N), io)
+    s = _dev(s)
+    length, new_starts = _length_ns(length, new_starts, B, T, r.device)
+    y = torch.empty_like(r)
+    new_s = torch.empty_like(s)
+    rc = lib.hiprwkv_wkv6_fwd(_stream(), _DT[io], _DT[s.dtype], B, T, H, N, _p(r), _p(k), _p(v), _p(w), _p(u), _p(s),
+                              _p(length), _p(new_starts), _p(y), _p(new_s), _flags(compat))
+    _lib.check(rc, "hiprwkv_wkv6_fwd")
+    return new_s, y
+
+
+def wkv6_bwd(r, k, v, w, u, s, length, new_starts, gy, gs_out=None, compat=True):
+    """Cotangents (gr, gk, gv, gw, gu, gs) of ``wkv6_fwd``; gu is summed over the batch here."""
+    lib = _lib.load()
+    io = r.dtype
+    B, T, H, N = r.shape
+    r, k, v, gy = (_dev(x, io) for x in (r, k, v, gy))
+    w = _dev(w.reshape(B, T, H, N), io)
+    u = _dev(u.reshape(H, N), io)
+    s = _dev(s)
+    gs_out = None if gs_out is None else _dev(gs_out, s.dtype)
+    length, new_starts = _length_ns(length, new_starts, B, T, r.device)
+    gr, gk, gv, gw = (torch.empty_like(r) for _ in range(4))
+    gu = torch.empty((B, H, N), dtype=torch.float32, device=r.device)
+    gs = torch.empty_like(s)
+    nbytes = lib.hiprwkv_wkv6_bwd_workspace_bytes(B, T, H, N)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=r.device)
+    rc = lib.hiprwkv_wkv6_bwd(_stream(), _DT[io], _DT[s.dtype], B, T, H, N, _p(r), _p(k), _p(v), _p(w), _p(u), _p(s),
+                              _p(length), _p(new_starts), _p(gy), _p(gs_out), _p(gr), _p(gk), _p(gv), _p(gw), _p(gu),
+                              _p(gs), _p(ws), nbytes, _flags(compat))
+    _lib.check(rc, "hiprwkv_wkv6_bwd")
+    return gr, gk, gv, gw, gu.sum(0).to(io), gs
+
+
+class _Wkv6(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, r, k, v, w, u, s, length, new_starts, compat):
+        new_s, y = wkv6_fwd(r, k, v, w, u, s, length, new_starts, compat)
+        ctx.compat = compat
+        ctx.shapes = (w.shape, u.shape)
+        ctx.save_for_backward(r, k, v, w, u, s, length, new_starts)
+        return new_s, y
+
+    @staticmethod
+    def backward(ctx, gs_out, gy):
+        r, k, v, w, u, s, length, new_starts = ctx.saved_tensors
+        if gy is None:
+            gy = torch.zeros_like(r)
+        gr, gk, gv, gw, gu, gs = wkv6_bwd(r, k, v, w, u, s, length, new_starts, gy, gs_out, ctx.compat)
+        return gr, gk, gv, gw.reshape(ctx.shapes[0]), gu.reshape(ctx.shapes[1]), gs, None, None, None
+
+
+def wkv6(r, k, v, w, u, s, length=None, new_starts=None, compat=True):
+    """Differentiable WKV6: returns (new_s, y)."""
+    B, T = r.shape[:2]
+    length, new_starts = _length_ns(length, new_starts, B, T, r.device)
+    return _Wkv6.apply(r, k, v, w, u, s, length, new_starts, compat)
+
+
+# ----------------------------------------------------------------------------- WKV4
+def wkv4_fwd(w_neg, u, k, v, s, length=None, new_starts=None, compat=True):
+    """w_neg = -exp(time_decay), u (C,); k,v (B,T,C); s (B,3,C).  Returns (new_s, wkv) -- receptance not applied."""
+    lib = _lib.load()
+    io = k.dtype
+    k, v, s, w_neg, u = (_dev(x, io) for x in (k, v, s, w_neg, u))
+    B, T, C = k.shape
+    assert s.shape == (B, 3, C) and w_neg.shape == (C,) and u.shape == (C,)
+    length, new_starts = _length_ns(length, new_starts, B, T, k.device)
+    y = torch.empty_like(k)
+    new_s = torch.empty_like(s)
+    rc = lib.hiprwkv_wkv4_fwd(_stream(), _DT[io], B, T, C, _p(w_neg), _p(u), _p(k), _p(v), _p(s), _p(length),
+                              _p(new_starts), _p(new_s), _p(y), _flags(compat))
+    _lib.check(rc, "hiprwkv_wkv4_fwd")
+    return new_s, y

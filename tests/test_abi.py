@@ -1,0 +1,66 @@
+"""CPU-only checks of the boundary: the library loads, exports every declared symbol, and refuses CPU tensors."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "hiprwkv.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(hiprwkv_\w+)\s*\(", text)))
+
+
+def test_header_declares_the_expected_entry_points():
+    syms = declared_symbols()
+    for need in ("hiprwkv_wkv7_fwd", "hiprwkv_wkv7_bwd", "hiprwkv_wkv6_fwd", "hiprwkv_wkv6_bwd", "hiprwkv_wkv4_fwd",
+                 "hiprwkv_last_error"):
+        assert need in syms
+
+
+def test_library_exports_every_declared_symbol():
+    from jaxrwkv_amd import _lib
+    lib = _lib.load()
+    for sym in declared_symbols():
+        assert hasattr(lib, sym), sym
+        assert sym in _lib.SIGNATURES, f"{sym} has no ctypes signature"
+    assert lib.hiprwkv_version() >= 100
+
+
+def test_argument_validation_without_gpu():
+    from jaxrwkv_amd import _lib
+    lib = _lib.load()
+    null = ctypes.c_void_p(0)
+    # head size other than 64 and null pointers are refused before anything is launched
+    rc = lib.hiprwkv_wkv7_fwd(null, 0, 0, 1, 8, 1, 32, *([null] * 12), 0)
+    assert rc == -1 and b"N=32" in lib.hiprwkv_last_error()
+    rc = lib.hiprwkv_wkv7_fwd(null, 0, 0, 1, 8, 1, 64, *([null] * 12), 0)
+    assert rc == -1 and b"null" in lib.hiprwkv_last_error()
+    rc = lib.hiprwkv_wkv6_fwd(null, 7, 0, 1, 8, 1, 64, *([null] * 10), 0)
+    assert rc == -1 and b"dtype" in lib.hiprwkv_last_error()
+    rc = lib.hiprwkv_wkv4_fwd(null, 0, 0, 8, 64, *([null] * 9), 0)
+    assert rc == -1
+    assert lib.hiprwkv_wkv7_bwd_workspace_bytes(2, 16, 2, 64) == 3 * 2 * 16 * 2 * 64 * 4
+    assert lib.hiprwkv_wkv6_bwd_workspace_bytes(2, 16, 2, 64) >= 2 * 16 * 2 * 64 * 4
+
+
+def test_cpu_tensors_are_refused_loudly():
+    from jaxrwkv_amd import _lib, ops
+    x = torch.zeros(1, 4, 1, 64)
+    with pytest.raises(_lib.HipRwkvError):
+        ops.wkv7_fwd(x, x, x, x, x, x, torch.zeros(1, 1, 64, 64))
+    with pytest.raises(_lib.HipRwkvError):
+        ops.wkv4_fwd(torch.zeros(8), torch.zeros(8), torch.zeros(1, 4, 8), torch.zeros(1, 4, 8), torch.zeros(1, 3, 8))
+
+
+def test_product_does_not_import_the_oracle():
+    pkg = os.path.join(ROOT, "jaxrwkv_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h", ".cpp")):
+                src = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in src, f"{f} mentions the oracle"
