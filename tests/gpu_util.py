@@ -29,11 +29,13 @@ def assert_close(name, got, ref, rtol=FP32_RTOL, atol=FP32_ATOL, scale_atol=Fals
 
 
 def tvd_of_projected(y_a, y_b, vocab=512, seed=0):
-    """Total-variation distance of softmax(y @ P) for a fixed random projection: the op-level proxy of 'logits TVD'."""
+    """Total-variation distance of softmax(groupnorm(y) @ P) for a fixed random projection P: the op-level proxy
+    of 'logits TVD' (the model applies a per-head group norm to y, rwkv7.py:263, before any projection)."""
     g = np.random.default_rng(seed)
     C = y_a.shape[-2] * y_a.shape[-1]
     P = g.standard_normal((C, vocab)) / np.sqrt(C)
     def sm(y):
+        y = (y - y.mean(-1, keepdims=True)) / np.sqrt(y.var(-1, keepdims=True) + 64e-5)
         z = y.reshape(y.shape[0], y.shape[1], C) @ P
         z = z - z.max(-1, keepdims=True)
         e = np.exp(z)
