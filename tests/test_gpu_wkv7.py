@@ -118,7 +118,8 @@ def test_bf16_io_against_float64_oracle():
     new_s, y, _ = run_fwd(x, torch.bfloat16, True)
     # y is rounded to bf16 on output: half an ulp = 2^-9 relative
     assert_close("y", y, ref_y, rtol=2.0 ** -8, atol=1e-3)
-    assert_close("new_s", new_s, ref_s)                   # fp32 state: the fp32 bar
+    # fp32 state out of the chunked MFMA kernel (operands fed as bf16 hi+lo pairs, ~16 mantissa bits)
+    assert_close("new_s", new_s, ref_s, rtol=1e-4, atol=1e-4, scale_atol=True)
     # bf16 bar: TVD of projected outputs below 1e-3, against the oracle's y rounded to the same output type
     tvd = tvd_of_projected(y, bf16_round(ref_y).astype(np.float64))
     assert tvd.max() < 1e-3, tvd.max()
