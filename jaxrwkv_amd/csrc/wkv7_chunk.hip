@@ -15,11 +15,15 @@
 // significant partial products are accumulated (hi.hi + hi.lo + lo.hi), which keeps ~16 mantissa bits; the
 // doubling chain of the inverse alone runs in single bf16 (its result is split again).  The K = 32 slots of one
 // MFMA hold two 16-token products side by side.  The state stays in fp32 accumulator registers for the whole
-// sequence, transposed (key x value tiles) so that accumulator registers can be reused directly as B operands.
+// sequence, transposed (key x value tiles), so that accumulator registers are reused directly as B operands.
 //
-// Work split: one workgroup per (sequence, head); wave q owns value rows 16q..16q+15 of the state.
-// new_starts inside a chunk are handled by restarting the cumulative decay and masking (rare, uniform branch).
-// `length` snapshots use a second set of masked update operands for the one chunk that holds token length-1.
+// Work split: one workgroup of 8 waves per (sequence, head).  Waves 0-3 are consumers: wave q owns value rows
+// 16q..16q+15 of the state and runs the S0-dependent part of every chunk.  Waves 4-7 are producers: producer p
+// prepares chunks p, p+4, p+8, ... (everything that does not depend on S0: decay scan, scaled operands, Gram
+// tiles, triangular inverse, operand transposes) into a ring of LDS slots, four chunk periods ahead of the
+// consumers.  One workgroup barrier per chunk period is the only synchronisation.
+// new_starts inside a chunk restart the cumulative decay and mask the Gram tiles (rare, uniform branch).
+// `length` snapshots use a second, masked set of update operands for the one chunk that holds token length-1.
 //
 // Range: the cumulative log decay inside a chunk is clamped at -80 so that 1/E_s stays finite in fp32.  A key
 // channel whose decay over at most 16 tokens falls below e^-80 (RWKV-7 models keep d >= 0.54 per token, i.e.
@@ -38,27 +42,31 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int CK = 16;            // tokens per chunk
 constexpr int RS = 72;            // row stride (bf16 elements) of the [token][64] LDS arrays: 144 B (16-byte aligned rows)
-constexpr int TS = 20;            // row stride of the [key][16 tokens] LDS arrays: 40 B
+constexpr int NPROD = 4;          // producer waves; a producer owns every NPROD-th chunk and has NPROD periods for it
+constexpr int RING = NPROD + 1;   // slots: a slot is rewritten no earlier than the period after it was consumed
 constexpr float LOG2E = 1.44269504088896340736f;
 constexpr float MIN_STEP_L2 = -1.0e4f;          // keeps the running sum finite
 constexpr float MIN_CUM_L2 = -80.0f * LOG2E;    // 2^MIN_CUM_L2 = e^-80
 
-// One chunk's operands as the consumers read them.
+// One chunk's operands as the consumers read them.  "lane-indexed" arrays hold, for every lane of the producer,
+// the 8 bytes that the same lane of a consumer loads: accumulator-layout registers (column lane%16, rows
+// 4*(lane/16)..+3) packed to bf16, which is exactly the A-operand layout (row lane%16, k-slots 4*(lane/16)..+3).
 struct __attribute__((aligned(16))) Slot {
-  uint16_t At[2][CK][RS];      // hi/lo of a_t.Ee_t, rows of tokens the entering state does not reach are zero
-  uint16_t Qt[2][CK][RS];      // hi/lo of r_t.E_t, same masking (+ rows whose y is defined as zero)
-  uint16_t BhT[2][64][TS];     // hi/lo of (b_s/E_s)^T, columns cut off from the chunk end by a reset are zero
-  uint16_t KhT[2][64][TS];
-  uint16_t SBhT[2][64][TS];    // same, masked for the state snapshot at token `length-1`
-  uint16_t SKhT[2][64][TS];
-  uint16_t V[CK][RS];          // raw v
-  uint2 Mt[4][2][64];          // T, Mka, Mbr, Mkr: hi/lo accumulator-layout registers, indexed by lane
+  uint16_t At[2][CK][RS];      // hi/lo of a_t.Ee_t; rows the entering state does not reach are zero
+  uint16_t Qt[2][CK][RS];      // hi/lo of r_t.E_t; same masking, plus rows whose y is defined as zero
+  uint2 BT[2][2][4][64];       // [bh|kh][hi|lo][key tile]: (b_s/E_s)^T, lane-indexed; masked for the chunk-end state
+  uint2 VT[4][64];             // v^T per value tile, lane-indexed
+  uint2 Mt[4][2][64];          // T, Mka, Mbr, Mkr: hi/lo, lane-indexed
   float gamma[64];             // E at the chunk end
-  float sgamma[64];            // E at the snapshot token
   int snap;                    // -1, or the in-chunk index of token length-1
   int keep_end;                // the entering state survives to the chunk end (no reset in the chunk)
   int keep_snap;               // the entering state survives to the snapshot token
   int pad;
+};
+// Update operands masked for the snapshot token; only one chunk per sequence needs them.
+struct __attribute__((aligned(16))) SnapSlot {
+  uint2 BT[2][2][4][64];
+  float gamma[64];
 };
 
 __device__ __forceinline__ f32x4_t mfma(const u32x4_t a, const u32x4_t b, f32x4_t c) {
@@ -68,6 +76,10 @@ __device__ __forceinline__ f32x4_t mfma(const u32x4_t a, const u32x4_t b, f32x4_
 __device__ __forceinline__ uint32_t pack_rn(float x0, float x1) {
   bf16x2_t p = {(__bf16)x0, (__bf16)x1};
   return __builtin_bit_cast(uint32_t, p);
+}
+// both values are exactly representable in bf16: keep the high halves
+__device__ __forceinline__ uint32_t pack_exact(float x0, float x1) {
+  return __builtin_amdgcn_perm(__float_as_uint(x1), __float_as_uint(x0), 0x07060302u);
 }
 
 // (x0, x1) -> packed truncated-bf16 hi parts and packed bf16 lo parts (x = hi + lo up to 2^-17 relative)
@@ -83,7 +95,7 @@ __device__ __forceinline__ float dpp0(float x) {  // lanes without a source read
 }
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// Per-chunk facts about new_starts, identical in every lane.
+// Per-chunk facts, identical in every lane.
 struct ChunkFlags {
   uint32_t ns;      // bit t: new_starts[c0+t], bit 16: new_starts[c0+16] (0 beyond T)
   int nvalid;       // tokens of this chunk that exist
@@ -93,10 +105,21 @@ struct ChunkFlags {
 
 __device__ __forceinline__ int seg_of(uint32_t ns, int t) { return __builtin_popcount(ns & ((2u << t) - 1u)); }
 
+__device__ __forceinline__ ChunkFlags chunk_flags(const Wkv7Args& A, int64_t b, int64_t c0, int64_t L, int lane) {
+  ChunkFlags F;
+  F.compat = (A.flags & 1u) != 0;
+  F.nvalid = (int)((A.T - c0 < CK) ? (A.T - c0) : CK);
+  F.snap = (L >= 1 && L - 1 >= c0 && L - 1 < c0 + CK) ? (int)(L - 1 - c0) : -1;
+  // lanes 0..16 fetch one flag each; the ballot makes the 17-bit mask uniform
+  bool mine = false;
+  if (A.ns != nullptr && lane <= CK && c0 + lane < A.T) mine = A.ns[(size_t)b * A.T + c0 + lane] != 0;
+  F.ns = (uint32_t)(__ballot(mine) & 0x1ffffull);
+  return F;
+}
+
 // ---------------------------------------------------------------------------------------------------- producer
-// One wave turns the raw r,w,k,v,a,b of a chunk into a Slot.  Lane (t = lane%16, g = lane/16) owns token t and the
-// keys {8g..8g+7} u {32+8g..32+8g+7}: exactly the A/B operand layout of the Gram MFMAs, and one 16-byte global load
-// per half.
+// Lane (t = lane%16, g = lane/16) owns token t and the keys {8g..8g+7} u {32+8g..32+8g+7}: exactly the A/B
+// operand layout of the Gram MFMAs (row/column = token, k-slots = keys), and one 16-byte global load per half.
 struct Raw {
   uint4 r[2], w[2], k[2], v[2], a[2], b[2];
 };
@@ -129,12 +152,36 @@ __device__ __forceinline__ void unpack16(const uint4 (&p)[2], float (&o)[16]) {
 // element e of a lane's 16 keys -> key index
 __device__ __forceinline__ int key_of(int g, int e) { return (e < 8) ? 8 * g + e : 32 + 8 * g + (e - 8); }
 
-__device__ __forceinline__ void produce(const Raw& x, const ChunkFlags& F, Slot* __restrict__ slot, int lane) {
-  const int t = lane & 15, g = lane >> 4;
+// Producer state carried from one period to the next (registers).
+struct Producer {
+  int lane;
+  u32x4_t sel[2];     // B operands that pick keys 16*(tile%2)..+15 out of a 32-key half: MFMA as a transposer
+  // stage 0 -> 1
+  float pa[16], pq[16], pk[16], pb[16];   // a.Ee, r.E, k/E, b/E
+  // stage 1 -> 2,3
+  u32x4_t at_h[2], at_l[2], qt_h[2], qt_l[2], kh_h[2], kh_l[2], bh_h[2], bh_l[2];
+  f32x4_t Mba, MbaT, Mka, Mbr, Mkr;
+};
+
+// stage 0: decay scan and scaled operands (fp32); v^T and the chunk-end decay go straight to the slot
+__device__ __forceinline__ void prod_stage0(Producer& P, const Raw& x, const ChunkFlags& F, Slot* __restrict__ slot,
+                                            SnapSlot* __restrict__ snap) {
+  const int lane = P.lane, t = lane & 15, g = lane >> 4;
   const bool valid = t < F.nvalid;
-  float fr[16], fk[16], fa[16], fb[16], E[16], Einv[16];
+  float fr[16], fk[16], fa[16], fb[16], E[16];
   unpack16(x.r, fr); unpack16(x.k, fk); unpack16(x.a, fa); unpack16(x.b, fb);
-  const bool slow = (F.ns != 0);
+  {
+    // transpose by MFMA: D[token][value of tile] = sum_k V[token][k] sel[k][value]; the accumulator layout of D
+    // (lane = value, registers = 4 consecutive tokens) is the B-operand layout the consumers need
+    const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int tile = 0; tile < 4; ++tile) {
+      const uint4 vr = x.v[tile >> 1];
+      const u32x4_t vop = {vr.x, vr.y, vr.z, vr.w};
+      const f32x4_t dv = mfma(vop, P.sel[tile & 1], zero4);
+      slot->VT[tile][lane] = make_uint2(pack_exact(dv[0], dv[1]), pack_exact(dv[2], dv[3]));
+    }
+  }
   {
     float fw[16];
     unpack16(x.w, fw);
@@ -149,99 +196,130 @@ __device__ __forceinline__ void produce(const Raw& x, const ChunkFlags& F, Slot*
       E[e] = l2;
     }
   }
-  int myseg = 0;
+  const bool slow = (F.ns & 0xffffu) != 0;
   if (slow) {
     // restart the cumulative decay at the last reset at or before this token
-    myseg = seg_of(F.ns, t);
     const uint32_t upto = F.ns & ((2u << t) - 1u) & 0xffffu;
     const int p = upto ? 31 - __builtin_clz(upto) : 0;   // position of that reset
     const int src = (lane & 48) | (p > 0 ? p - 1 : 0);
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
       const float base = __shfl(E[e], src, 64);
-      if (upto != 0 && p > 0) E[e] -= base;
+      if (p > 0) E[e] -= base;
     }
     if ((F.ns >> t) & 1u) {
 #pragma unroll
-      for (int e = 0; e < 16; ++e) fa[e] = 0.f;
+      for (int e = 0; e < 16; ++e) fa[e] = 0.f;   // the state entering a reset token is zero: sa = 0
     }
   }
-  float Ee[16];
 #pragma unroll
   for (int e = 0; e < 16; ++e) {
     const float l2 = fmaxf(E[e], MIN_CUM_L2);
-    E[e] = exp2_fast(l2);
-    Einv[e] = exp2_fast(-l2);
+    const float Ev = exp2_fast(l2), Einv = exp2_fast(-l2);
     // exclusive: value of the previous token; 1 for the first token of the chunk
-    Ee[e] = __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(1.0f), __float_as_int(E[e]), 0x111, 0xf, 0xf, false));
+    const float Ee = __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(1.0f), __float_as_int(Ev), 0x111, 0xf, 0xf, false));
+    P.pa[e] = fa[e] * Ee;      // at a reset token a is zero, whatever Ee holds
+    P.pq[e] = fr[e] * Ev;
+    P.pk[e] = fk[e] * Einv;
+    P.pb[e] = fb[e] * Einv;
+    E[e] = Ev;
   }
-  if (slow && ((F.ns >> t) & 1u)) {
+  if (t == 15) {
 #pragma unroll
-    for (int e = 0; e < 16; ++e) Ee[e] = 1.f;   // (a is zero there anyway)
+    for (int hf = 0; hf < 2; ++hf) {
+      float* gp = &slot->gamma[8 * g + 32 * hf];
+      *reinterpret_cast<float4*>(gp) = make_float4(E[8 * hf], E[8 * hf + 1], E[8 * hf + 2], E[8 * hf + 3]);
+      *reinterpret_cast<float4*>(gp + 4) = make_float4(E[8 * hf + 4], E[8 * hf + 5], E[8 * hf + 6], E[8 * hf + 7]);
+    }
   }
-  // scaled operands, split into hi/lo bf16 pairs: dword j of half hf covers elements 8*hf + 2j, 8*hf + 2j + 1
-  u32x4_t at_h[2], at_l[2], qt_h[2], qt_l[2], kh_h[2], kh_l[2], bh_h[2], bh_l[2];
+  if (t == F.snap) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) snap->gamma[key_of(g, e)] = E[e];
+  }
+}
+
+// stage 1: hi/lo split and the five Gram tiles
+__device__ __forceinline__ void prod_stage1(Producer& P) {
 #pragma unroll
   for (int hf = 0; hf < 2; ++hf) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int e = 8 * hf + 2 * j;
       uint32_t hi, lo;
-      split2(fa[e] * Ee[e], fa[e + 1] * Ee[e + 1], hi, lo); at_h[hf][j] = hi; at_l[hf][j] = lo;
-      split2(fr[e] * E[e], fr[e + 1] * E[e + 1], hi, lo);   qt_h[hf][j] = hi; qt_l[hf][j] = lo;
-      split2(fk[e] * Einv[e], fk[e + 1] * Einv[e + 1], hi, lo); kh_h[hf][j] = hi; kh_l[hf][j] = lo;
-      split2(fb[e] * Einv[e], fb[e + 1] * Einv[e + 1], hi, lo); bh_h[hf][j] = hi; bh_l[hf][j] = lo;
+      split2(P.pa[e], P.pa[e + 1], hi, lo); P.at_h[hf][j] = hi; P.at_l[hf][j] = lo;
+      split2(P.pq[e], P.pq[e + 1], hi, lo); P.qt_h[hf][j] = hi; P.qt_l[hf][j] = lo;
+      split2(P.pk[e], P.pk[e + 1], hi, lo); P.kh_h[hf][j] = hi; P.kh_l[hf][j] = lo;
+      split2(P.pb[e], P.pb[e + 1], hi, lo); P.bh_h[hf][j] = hi; P.bh_l[hf][j] = lo;
     }
   }
-  // ---- Gram tiles (accumulator layout: lane holds column n = lane%16, rows m = 4g..4g+3)
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
-  auto gram = [&](const u32x4_t (&ah)[2], const u32x4_t (&al)[2], const u32x4_t (&bh)[2], const u32x4_t (&bl)[2]) {
-    f32x4_t acc = zero4;
+  f32x4_t Mba = zero4, MbaT = zero4, Mka = zero4, Mbr = zero4, Mkr = zero4;
+  // accumulator layout: lane holds column n = lane%16, rows m = 4g..4g+3.  Five independent chains, interleaved.
 #pragma unroll
-    for (int hf = 0; hf < 2; ++hf) {
-      acc = mfma(ah[hf], bh[hf], acc);
-      acc = mfma(ah[hf], bl[hf], acc);
-      acc = mfma(al[hf], bh[hf], acc);
+  for (int hf = 0; hf < 2; ++hf) {
+#pragma unroll
+    for (int part = 0; part < 3; ++part) {
+      const u32x4_t bA = part == 2 ? P.bh_l[hf] : P.bh_h[hf], kA = part == 2 ? P.kh_l[hf] : P.kh_h[hf];
+      const u32x4_t aA = part == 2 ? P.at_l[hf] : P.at_h[hf];
+      const u32x4_t aB = part == 1 ? P.at_l[hf] : P.at_h[hf], qB = part == 1 ? P.qt_l[hf] : P.qt_h[hf];
+      const u32x4_t bB = part == 1 ? P.bh_l[hf] : P.bh_h[hf];
+      Mba = mfma(bA, aB, Mba);     // [s][t] = bh_s . at_t
+      MbaT = mfma(aA, bB, MbaT);   // [t][s]
+      Mka = mfma(kA, aB, Mka);     // [s][t] = kh_s . at_t
+      Mbr = mfma(bA, qB, Mbr);     // [s][t] = bh_s . qt_t
+      Mkr = mfma(kA, qB, Mkr);     // [s][t] = kh_s . qt_t
     }
-    return acc;
-  };
-  f32x4_t Mba = gram(bh_h, bh_l, at_h, at_l);    // [s][t]
-  f32x4_t MbaT = gram(at_h, at_l, bh_h, bh_l);   // [t][s]
-  f32x4_t Mka = gram(kh_h, kh_l, at_h, at_l);    // [s][t]
-  f32x4_t Mbr = gram(bh_h, bh_l, qt_h, qt_l);    // [s][t]
-  f32x4_t Mkr = gram(kh_h, kh_l, qt_h, qt_l);    // [s][t]
-  const int n = t;  // accumulator column of this lane
-  const bool dropy = F.compat && ((F.ns >> (n + 1)) & 1u);   // y[n] is defined as zero
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int m = 4 * g + i;
-    bool same = true;
-    if (slow) same = seg_of(F.ns, m) == seg_of(F.ns, n);
-    const bool lt = (m < n) && same, le = (m <= n) && same, gt = (m > n) && same;
-    Mba[i] = lt ? Mba[i] : 0.f;
-    Mka[i] = lt ? Mka[i] : 0.f;
-    Mbr[i] = (le && !dropy) ? Mbr[i] : 0.f;
-    Mkr[i] = (le && !dropy) ? Mkr[i] : 0.f;
-    MbaT[i] = gt ? MbaT[i] : 0.f;   // [t = m][s = n], s < t
   }
-  // ---- T = (I - Mba)^{-1} = (I + M^8)(I + M^4)(I + M^2)(I + M), single-bf16 operands
+  P.Mba = Mba; P.MbaT = MbaT; P.Mka = Mka; P.Mbr = Mbr; P.Mkr = Mkr;
+}
+
+// stage 2: triangular masks, T = (I - Mba)^{-1}, park T / Mka / Mbr / Mkr
+__device__ __forceinline__ void prod_stage2(Producer& P, const ChunkFlags& F, Slot* __restrict__ slot) {
+  const int lane = P.lane, n = lane & 15, g = lane >> 4;
+  const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+  f32x4_t Mba = P.Mba, MbaT = P.MbaT, Mka = P.Mka, Mbr = P.Mbr, Mkr = P.Mkr;
+  const bool slow = F.ns != 0;
+  if (!slow) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = 4 * g + i;
+      Mba[i] = (m < n) ? Mba[i] : 0.f;
+      Mka[i] = (m < n) ? Mka[i] : 0.f;
+      Mbr[i] = (m <= n) ? Mbr[i] : 0.f;
+      Mkr[i] = (m <= n) ? Mkr[i] : 0.f;
+      MbaT[i] = (m > n) ? MbaT[i] : 0.f;   // [t = m][s = n], s < t
+    }
+  } else {
+    const bool dropy = F.compat && ((F.ns >> (n + 1)) & 1u);   // y[n] is defined as zero
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = 4 * g + i;
+      const bool same = seg_of(F.ns, m) == seg_of(F.ns, n);
+      const bool lt = (m < n) && same, le = (m <= n) && same, gt = (m > n) && same;
+      Mba[i] = lt ? Mba[i] : 0.f;
+      Mka[i] = lt ? Mka[i] : 0.f;
+      Mbr[i] = (le && !dropy) ? Mbr[i] : 0.f;
+      Mkr[i] = (le && !dropy) ? Mkr[i] : 0.f;
+      MbaT[i] = gt ? MbaT[i] : 0.f;
+    }
+  }
+  // T = (I + M^8)(I + M^4)(I + M^2)(I + M), single-bf16 operands
   auto single = [&](const f32x4_t d) {
     u32x4_t o = {pack_rn(d[0], d[1]), pack_rn(d[2], d[3]), 0u, 0u};
     return o;
   };
-  f32x4_t P = Mba;
+  f32x4_t Pm = Mba;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) P[i] += (4 * g + i == n) ? 1.f : 0.f;
+  for (int i = 0; i < 4; ++i) Pm[i] += (4 * g + i == n) ? 1.f : 0.f;
   f32x4_t Mp = Mba, MpT = MbaT;
 #pragma unroll
   for (int lvl = 0; lvl < 3; ++lvl) {
     const u32x4_t om = single(Mp), omt = single(MpT);
-    const f32x4_t M2 = mfma(omt, om, zero4);     // (M^2)[s][t]  : A rows from the transpose, B cols from M
-    const f32x4_t M2T = mfma(om, omt, zero4);    // (M^2)^T[t][s]
-    Mp = M2; MpT = M2T;
-    P = mfma(single(MpT), single(P), P);         // P += M^(2^(lvl+1)) P
+    const f32x4_t M2T = mfma(om, omt, zero4);      // (M^2)^T[t][s]
+    if (lvl < 2) Mp = mfma(omt, om, zero4);        // (M^2)[s][t]: A rows from the transpose, B columns from M
+    MpT = M2T;
+    Pm = mfma(single(MpT), single(Pm), Pm);        // P += M^(2^(lvl+1)) P
   }
-  // ---- park everything in the slot
   uint32_t hi0, lo0, hi1, lo1;
   auto park = [&](int which, const f32x4_t d) {
     split2(d[0], d[1], hi0, lo0);
@@ -249,56 +327,74 @@ __device__ __forceinline__ void produce(const Raw& x, const ChunkFlags& F, Slot*
     slot->Mt[which][0][lane] = make_uint2(hi0, hi1);
     slot->Mt[which][1][lane] = make_uint2(lo0, lo1);
   };
-  park(0, P); park(1, Mka); park(2, Mbr); park(3, Mkr);
+  park(0, Pm); park(1, Mka); park(2, Mbr); park(3, Mkr);
+}
 
-  const bool s0_reaches = !slow || myseg == 0;           // the entering state reaches this token
-  const bool q_keep = s0_reaches && !(F.compat && ((F.ns >> (t + 1)) & 1u));
+// stage 3: operands the consumers read through LDS: At, Qt (row-major), transposed bh / kh, flags
+__device__ __forceinline__ void prod_stage3(Producer& P, const ChunkFlags& F, Slot* __restrict__ slot,
+                                            SnapSlot* __restrict__ snap) {
+  const int lane = P.lane, t = lane & 15, g = lane >> 4;
+  const bool slow = F.ns != 0;
+  const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
   const u32x4_t z4 = {0u, 0u, 0u, 0u};
+  int lastseg = 0;
+  bool s0_reaches = true, q_keep = true;
+  uint32_t keep_upd = 0xffffu;       // tokens that still contribute to the chunk-end state
+  if (slow) {
+    lastseg = seg_of(F.ns, 15);
+    s0_reaches = seg_of(F.ns, t) == 0;                             // the entering state reaches this token
+    q_keep = s0_reaches && !(F.compat && ((F.ns >> (t + 1)) & 1u));
+    const uint32_t resets = F.ns & 0xffffu;
+    // tokens from the last reset on
+    keep_upd = resets ? (0xffffu & ~((1u << (31 - __builtin_clz(resets))) - 1u)) : 0xffffu;
+  }
 #pragma unroll
   for (int hf = 0; hf < 2; ++hf) {
     const int col = 8 * g + 32 * hf;
-    *reinterpret_cast<u32x4_t*>(&slot->At[0][t][col]) = s0_reaches ? at_h[hf] : z4;
-    *reinterpret_cast<u32x4_t*>(&slot->At[1][t][col]) = s0_reaches ? at_l[hf] : z4;
-    *reinterpret_cast<u32x4_t*>(&slot->Qt[0][t][col]) = q_keep ? qt_h[hf] : z4;
-    *reinterpret_cast<u32x4_t*>(&slot->Qt[1][t][col]) = q_keep ? qt_l[hf] : z4;
-    *reinterpret_cast<uint4*>(&slot->V[t][col]) = x.v[hf];
+    *reinterpret_cast<u32x4_t*>(&slot->At[0][t][col]) = s0_reaches ? P.at_h[hf] : z4;
+    *reinterpret_cast<u32x4_t*>(&slot->At[1][t][col]) = s0_reaches ? P.at_l[hf] : z4;
+    *reinterpret_cast<u32x4_t*>(&slot->Qt[0][t][col]) = q_keep ? P.qt_h[hf] : z4;
+    *reinterpret_cast<u32x4_t*>(&slot->Qt[1][t][col]) = q_keep ? P.qt_l[hf] : z4;
   }
-  // transposed update operands: token t contributes to the chunk-end state iff no reset lies after it
-  const int lastseg = slow ? seg_of(F.ns, 15) : 0;
-  const bool upd_keep = !slow || myseg == lastseg;
-  bool snap_keep = false;
-  if (F.snap >= 0) snap_keep = (t <= F.snap) && (!slow || myseg == seg_of(F.ns, F.snap));
-#pragma unroll
-  for (int hf = 0; hf < 2; ++hf) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-#pragma unroll
-      for (int o = 0; o < 2; ++o) {
-        const int key = 8 * g + 32 * hf + 2 * j + o;
-        const uint16_t bhh = (uint16_t)(o ? bh_h[hf][j] >> 16 : bh_h[hf][j] & 0xffffu);
-        const uint16_t bhl = (uint16_t)(o ? bh_l[hf][j] >> 16 : bh_l[hf][j] & 0xffffu);
-        const uint16_t khh = (uint16_t)(o ? kh_h[hf][j] >> 16 : kh_h[hf][j] & 0xffffu);
-        const uint16_t khl = (uint16_t)(o ? kh_l[hf][j] >> 16 : kh_l[hf][j] & 0xffffu);
-        slot->BhT[0][key][t] = upd_keep ? bhh : (uint16_t)0;
-        slot->BhT[1][key][t] = upd_keep ? bhl : (uint16_t)0;
-        slot->KhT[0][key][t] = upd_keep ? khh : (uint16_t)0;
-        slot->KhT[1][key][t] = upd_keep ? khl : (uint16_t)0;
-        if (F.snap >= 0) {
-          slot->SBhT[0][key][t] = snap_keep ? bhh : (uint16_t)0;
-          slot->SBhT[1][key][t] = snap_keep ? bhl : (uint16_t)0;
-          slot->SKhT[0][key][t] = snap_keep ? khh : (uint16_t)0;
-          slot->SKhT[1][key][t] = snap_keep ? khl : (uint16_t)0;
-        }
-      }
+  // transposes by MFMA: D[token][key of tile] = sum_k X[token][k] sel[k][key]; the accumulator layout of D
+  // (lane = key, registers = 4 consecutive tokens) is the A-operand layout of the state update
+  uint32_t keep_snap = 0;
+  if (F.snap >= 0) {
+    keep_snap = (2u << F.snap) - 1u;
+    if (slow) {
+      const uint32_t upto = F.ns & keep_snap & 0xffffu;
+      if (upto) keep_snap &= ~((1u << (31 - __builtin_clz(upto))) - 1u);
     }
   }
-  if (t == 15) {
+  auto masked_pack = [&](const f32x4_t d, uint32_t keep) {
+    const uint32_t bits = keep >> (4 * g);
+    const float d0 = (bits & 1u) ? d[0] : 0.f, d1 = (bits & 2u) ? d[1] : 0.f;
+    const float d2 = (bits & 4u) ? d[2] : 0.f, d3 = (bits & 8u) ? d[3] : 0.f;
+    return make_uint2(pack_exact(d0, d1), pack_exact(d2, d3));
+  };
 #pragma unroll
-    for (int e = 0; e < 16; ++e) slot->gamma[key_of(g, e)] = E[e];
-  }
-  if (t == F.snap) {
-#pragma unroll
-    for (int e = 0; e < 16; ++e) slot->sgamma[key_of(g, e)] = E[e];
+  for (int tile = 0; tile < 4; ++tile) {
+    const int hf = tile >> 1;
+    const u32x4_t sel = P.sel[tile & 1];
+    const f32x4_t dbh = mfma(P.bh_h[hf], sel, zero4), dbl = mfma(P.bh_l[hf], sel, zero4);
+    const f32x4_t dkh = mfma(P.kh_h[hf], sel, zero4), dkl = mfma(P.kh_l[hf], sel, zero4);
+    if (keep_upd == 0xffffu) {
+      slot->BT[0][0][tile][lane] = make_uint2(pack_exact(dbh[0], dbh[1]), pack_exact(dbh[2], dbh[3]));
+      slot->BT[0][1][tile][lane] = make_uint2(pack_exact(dbl[0], dbl[1]), pack_exact(dbl[2], dbl[3]));
+      slot->BT[1][0][tile][lane] = make_uint2(pack_exact(dkh[0], dkh[1]), pack_exact(dkh[2], dkh[3]));
+      slot->BT[1][1][tile][lane] = make_uint2(pack_exact(dkl[0], dkl[1]), pack_exact(dkl[2], dkl[3]));
+    } else {
+      slot->BT[0][0][tile][lane] = masked_pack(dbh, keep_upd);
+      slot->BT[0][1][tile][lane] = masked_pack(dbl, keep_upd);
+      slot->BT[1][0][tile][lane] = masked_pack(dkh, keep_upd);
+      slot->BT[1][1][tile][lane] = masked_pack(dkl, keep_upd);
+    }
+    if (F.snap >= 0) {
+      snap->BT[0][0][tile][lane] = masked_pack(dbh, keep_snap);
+      snap->BT[0][1][tile][lane] = masked_pack(dbl, keep_snap);
+      snap->BT[1][0][tile][lane] = masked_pack(dkh, keep_snap);
+      snap->BT[1][1][tile][lane] = masked_pack(dkl, keep_snap);
+    }
   }
   if (lane == 0) {
     slot->snap = F.snap;
@@ -317,8 +413,8 @@ struct Consumer {
 
 __device__ __forceinline__ uint2 lds8(const uint16_t* p) { return *reinterpret_cast<const uint2*>(p); }
 
-__device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ slot, const Wkv7Args& A, int64_t b,
-                                        int64_t h, int64_t c0, int nvalid, bool q2drop) {
+__device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ slot, const SnapSlot* __restrict__ snapslot,
+                                        const Wkv7Args& A, int64_t b, int64_t h, int64_t c0, int nvalid, bool q2drop) {
   const int lane = C.lane, n = lane & 15, g = lane >> 4;
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
   // B operands from the state: MFMA j contracts over the keys of tiles 2j and 2j+1
@@ -342,18 +438,18 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const u32x4_t ah = rows(slot->At[0], j), al = rows(slot->At[1], j);
-    W = mfma(ah, Sh[j], W);
-    W = mfma(ah, Sl[j], W);
-    W = mfma(al, Sh[j], W);
     const u32x4_t qh = rows(slot->Qt[0], j), ql = rows(slot->Qt[1], j);
+    W = mfma(ah, Sh[j], W);
     Y = mfma(qh, Sh[j], Y);
+    W = mfma(ah, Sl[j], W);
     Y = mfma(qh, Sl[j], Y);
+    W = mfma(al, Sh[j], W);
     Y = mfma(ql, Sh[j], Y);
   }
   // v of the four tokens 4g..4g+3 for this lane's value column
   const int val = 16 * C.q + n;
-  const uint32_t v01 = (uint32_t)slot->V[4 * g][val] | ((uint32_t)slot->V[4 * g + 1][val] << 16);
-  const uint32_t v23 = (uint32_t)slot->V[4 * g + 2][val] | ((uint32_t)slot->V[4 * g + 3][val] << 16);
+  const uint2 vt = slot->VT[C.q][lane];
+  const uint32_t v01 = vt.x, v23 = vt.y;
   const uint2 Th = slot->Mt[0][0][lane], Tl = slot->Mt[0][1][lane];
   const uint2 Kah = slot->Mt[1][0][lane], Kal = slot->Mt[1][1][lane];
   const uint2 Brh = slot->Mt[2][0][lane], Brl = slot->Mt[2][1][lane];
@@ -382,24 +478,12 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
     Y = mfma(a2, bLV, Y);
     Y = mfma(a3, bV0, Y);                     // Y^T += Mbr^T SA^T + Mkr^T V^T
   }
-  // outputs: register i is token 4g+i, lanes n = 16 consecutive values
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int tt = 4 * g + i;
-    if (tt < nvalid) {
-      const size_t off = (((size_t)b * A.T + c0 + tt) * A.H + h) * 64 + val;
-      reinterpret_cast<uint16_t*>(A.out)[off] = f32_to_bf16(Y[i]);
-      if (A.sa != nullptr) A.sa[off] = SA[i];
-    }
-  }
   // state update (and the snapshot for `length`), tile by tile: rows = keys
-  auto update = [&](const uint16_t (*bT)[64][TS], const uint16_t (*kT)[64][TS], const float* gam, bool keep,
-                    f32x4_t (&out)[4]) {
+  auto update = [&](const uint2 (*bt)[2][4][64], const float* gam, bool keep, f32x4_t (&out)[4]) {
 #pragma unroll
     for (int tile = 0; tile < 4; ++tile) {
-      const int key = 16 * tile + n;
-      const uint2 bh = lds8(&bT[0][key][4 * g]), bl = lds8(&bT[1][key][4 * g]);
-      const uint2 kh = lds8(&kT[0][key][4 * g]), kl = lds8(&kT[1][key][4 * g]);
+      const uint2 bh = bt[0][0][tile][lane], bl = bt[0][1][tile][lane];
+      const uint2 kh = bt[1][0][tile][lane], kl = bt[1][1][tile][lane];
       const u32x4_t a1 = {bh.x, bh.y, bl.x, bl.y}, a2 = {bh.x, bh.y, kh.x, kh.y}, a3 = {kl.x, kl.y, 0u, 0u};
       f32x4_t acc = keep ? C.S[tile] : zero4;
       acc = mfma(a1, bSS, acc);
@@ -412,7 +496,7 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
   };
   if (slot->snap >= 0) {
     f32x4_t snap[4];
-    update(slot->SBhT, slot->SKhT, slot->sgamma, slot->keep_snap != 0, snap);
+    update(snapslot->BT, snapslot->gamma, slot->keep_snap != 0, snap);
 #pragma unroll
     for (int tile = 0; tile < 4; ++tile) {
       const size_t off = (((size_t)b * A.H + h) * 64 + val) * 64 + 16 * tile + 4 * g;
@@ -425,7 +509,17 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
       }
     }
   }
-  update(slot->BhT, slot->KhT, slot->gamma, slot->keep_end != 0, C.S);
+  update(slot->BT, slot->gamma, slot->keep_end != 0, C.S);
+  // outputs: register i is token 4g+i, lanes n = 16 consecutive values
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int tt = 4 * g + i;
+    if (tt < nvalid) {
+      const size_t off = (((size_t)b * A.T + c0 + tt) * A.H + h) * 64 + val;
+      reinterpret_cast<uint16_t*>(A.out)[off] = f32_to_bf16(Y[i]);
+      if (A.sa != nullptr) A.sa[off] = SA[i];
+    }
+  }
 }
 
 __device__ __forceinline__ void load_state(Consumer& C, const Wkv7Args& A, int64_t b, int64_t h) {
@@ -459,59 +553,81 @@ __device__ __forceinline__ void store_state0(const Consumer& C, const Wkv7Args& 
   }
 }
 
-__device__ __forceinline__ ChunkFlags chunk_flags(const Wkv7Args& A, int64_t b, int64_t c0, int64_t L) {
-  ChunkFlags F;
-  F.compat = (A.flags & 1u) != 0;
-  F.nvalid = (int)((A.T - c0 < CK) ? (A.T - c0) : CK);
-  F.snap = (L >= 1 && L - 1 >= c0 && L - 1 < c0 + CK) ? (int)(L - 1 - c0) : -1;
-  // lanes 0..16 fetch one flag each; the ballot makes the 17-bit mask uniform
-  const int lane = threadIdx.x & 63;
-  bool mine = false;
-  if (A.ns != nullptr && lane <= CK && c0 + lane < A.T) mine = A.ns[(size_t)b * A.T + c0 + lane] != 0;
-  F.ns = (uint32_t)(__ballot(mine) & 0x1ffffull);
-  return F;
-}
-
 }  // namespace
 
-// ------------------------------------------------------------------ kernel A: every wave prepares its own chunk copy
-// No cross-wave synchronisation: each of the four waves of a head runs producer and consumer back to back on a
-// private Slot.  Simple and self-contained; the specialised kernel below shares the producer work instead.
-__global__ __launch_bounds__(256) void wkv7_chunk_fwd_private_kernel(Wkv7Args A) {
+// Barrier schedule (period k ends with barrier k; every wave executes nchunks + NPROD barriers):
+//   producer p works on chunk c = p + NPROD*m during periods c .. c+NPROD-1, one stage per period;
+//   consumers work on chunk c during period c + NPROD.
+// Slot c % RING is rewritten from period c on; its previous chunk c - RING was consumed in period c - 1.
+__global__ __launch_bounds__(512) void wkv7_chunk_fwd_kernel(Wkv7Args A) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
+  Slot* slots = reinterpret_cast<Slot*>(smem_raw);
+  SnapSlot* snapslot = reinterpret_cast<SnapSlot*>(smem_raw + RING * sizeof(Slot));
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
-  Slot* slot = reinterpret_cast<Slot*>(smem_raw) + wave;
   const int64_t b = blockIdx.x / A.H, h = blockIdx.x % A.H;
   int64_t L = A.length ? (int64_t)A.length[b] : A.T;
   L = L < A.T ? L : A.T;
-  const bool q2drop = (A.flags & 1u) && L < A.T && A.ns != nullptr && A.ns[b * A.T + L] != 0;
-  Consumer C;
-  C.q = wave;
-  C.lane = lane;
-  load_state(C, A, b, h);
-  if (L == 0) store_state0(C, A, b, h, q2drop);
   const int64_t nchunks = (A.T + CK - 1) / CK;
-  Raw raw;
-  load_raw(raw, A, b, h, 0, lane);
-  for (int64_t c = 0; c < nchunks; ++c) {
-    const int64_t c0 = c * CK;
-    const ChunkFlags F = chunk_flags(A, b, c0, L);
-    produce(raw, F, slot, lane);
-    if (c + 1 < nchunks) load_raw(raw, A, b, h, c0 + CK, lane);
-    __builtin_amdgcn_s_waitcnt(0xc07f);      // lgkmcnt(0): this wave's LDS writes have landed
-    __builtin_amdgcn_wave_barrier();
-    consume(C, slot, A, b, h, c0, F.nvalid, q2drop);
-    __builtin_amdgcn_wave_barrier();
+
+  if (wave < 4) {
+    const bool q2drop = (A.flags & 1u) && L < A.T && A.ns != nullptr && A.ns[b * A.T + L] != 0;
+    Consumer C;
+    C.q = wave;
+    C.lane = lane;
+    load_state(C, A, b, h);
+    if (L == 0) store_state0(C, A, b, h, q2drop);
+    for (int i = 0; i < NPROD; ++i) __syncthreads();
+    for (int64_t c = 0; c < nchunks; ++c) {
+      const int64_t c0 = c * CK;
+      const int nvalid = (int)((A.T - c0 < CK) ? (A.T - c0) : CK);
+      consume(C, &slots[c % RING], snapslot, A, b, h, c0, nvalid, q2drop);
+      __syncthreads();
+    }
+  } else {
+    const int p = wave - 4;
+    Producer P;
+    P.lane = lane;
+    {
+      // sel[x]: k-slot (g, jj) of a 32-key half stands for key 8g + jj; column n of tile x is key 16x + n
+      const int n = lane & 15, g = lane >> 4;
+#pragma unroll
+      for (int x = 0; x < 2; ++x) {
+        const int jj = 16 * x + n - 8 * g;
+        u32x4_t s = {0u, 0u, 0u, 0u};
+        if (jj >= 0 && jj < 8) s[jj >> 1] = (jj & 1) ? 0x3f800000u : 0x00003f80u;
+        P.sel[x] = s;
+      }
+    }
+    for (int i = 0; i < p; ++i) __syncthreads();
+    int64_t done = p;
+    Raw raw;
+    if (p < nchunks) load_raw(raw, A, b, h, (int64_t)p * CK, lane);
+    for (int64_t c = p; c < nchunks; c += NPROD) {
+      const int64_t c0 = c * CK;
+      const ChunkFlags F = chunk_flags(A, b, c0, L, lane);
+      Slot* slot = &slots[c % RING];
+      prod_stage0(P, raw, F, slot, snapslot);
+      __syncthreads();
+      prod_stage1(P);
+      __syncthreads();
+      if (c + NPROD < nchunks) load_raw(raw, A, b, h, c0 + NPROD * CK, lane);   // needed two periods from now
+      prod_stage2(P, F, slot);
+      __syncthreads();
+      prod_stage3(P, F, slot, snapslot);
+      __syncthreads();
+      done += NPROD;
+    }
+    for (int64_t i = done; i < nchunks + NPROD; ++i) __syncthreads();
   }
 }
 
 hipError_t launch_wkv7_chunk_fwd(const Wkv7Args& A, hipStream_t stream) {
-  const size_t smem = 4 * sizeof(Slot);
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(wkv7_chunk_fwd_private_kernel),
+  const size_t smem = RING * sizeof(Slot) + sizeof(SnapSlot);
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(wkv7_chunk_fwd_kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(wkv7_chunk_fwd_private_kernel, dim3((unsigned)(A.B * A.H)), dim3(256), smem, stream, A);
+  hipLaunchKernelGGL(wkv7_chunk_fwd_kernel, dim3((unsigned)(A.B * A.H)), dim3(512), smem, stream, A);
   return hipGetLastError();
 }
 
