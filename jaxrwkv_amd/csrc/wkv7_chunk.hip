@@ -21,7 +21,10 @@
 // 16q..16q+15 of the state and runs the S0-dependent part of every chunk.  Waves 4-7 are producers: producer p
 // prepares chunks p, p+4, p+8, ... (everything that does not depend on S0: decay scan, scaled operands, Gram
 // tiles, triangular inverse, operand transposes) into a ring of LDS slots, four chunk periods ahead of the
-// consumers.  One workgroup barrier per chunk period is the only synchronisation.
+// consumers.  Synchronisation is a pair of LDS sequence numbers per slot: `ready` (set by the producer when a
+// chunk is complete) and `consumed` (one per consumer wave, set when it has read the slot for the last time).
+// Waiting is a bounded poll, so that a broken hand-shake ends the kernel (with wrong results) instead of
+// hanging the GPU.
 // new_starts inside a chunk restart the cumulative decay and mask the Gram tiles (rare, uniform branch).
 // `length` snapshots use a second, masked set of update operands for the one chunk that holds token length-1.
 //
@@ -42,8 +45,10 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int CK = 16;            // tokens per chunk
 constexpr int RS = 72;            // row stride (bf16 elements) of the [token][64] LDS arrays: 144 B (16-byte aligned rows)
-constexpr int NPROD = 4;          // producer waves; a producer owns every NPROD-th chunk and has NPROD periods for it
-constexpr int RING = NPROD + 1;   // slots: a slot is rewritten no earlier than the period after it was consumed
+constexpr int NPROD = 4;          // producer waves; producer p owns chunks p, p + NPROD, ...
+constexpr int NCONS = 4;          // consumer waves, one per 16 value rows
+constexpr int RING = 6;           // slots in flight
+constexpr int SPIN_LIMIT = 1 << 16;   // polls before a waiter gives up (milliseconds; a healthy wait is microseconds)
 constexpr float LOG2E = 1.44269504088896340736f;
 constexpr float MIN_STEP_L2 = -1.0e4f;          // keeps the running sum finite
 constexpr float MIN_CUM_L2 = -80.0f * LOG2E;    // 2^MIN_CUM_L2 = e^-80
@@ -68,6 +73,27 @@ struct __attribute__((aligned(16))) SnapSlot {
   uint2 BT[2][2][4][64];
   float gamma[64];
 };
+// Hand-shake words.  ready[s] = c + 1 once chunk c is complete in slot s; consumed[q][s] = c + 1 once consumer
+// q no longer reads chunk c in slot s.
+struct __attribute__((aligned(16))) Sync {
+  int ready[8];
+  int consumed[NCONS][8];
+};
+
+__device__ __forceinline__ void wait_ready(const Sync* sy, int slot, int want) {
+  for (int spin = 0; spin < SPIN_LIMIT; ++spin) {
+    if (__hip_atomic_load(&sy->ready[slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) == want) return;
+    __builtin_amdgcn_s_sleep(1);
+  }
+}
+__device__ __forceinline__ void wait_consumed(const Sync* sy, int slot, int want, int lane) {
+  for (int spin = 0; spin < SPIN_LIMIT; ++spin) {
+    int seen = want;
+    if (lane < NCONS) seen = __hip_atomic_load(&sy->consumed[lane][slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (__ballot(seen < want) == 0ull) return;
+    __builtin_amdgcn_s_sleep(1);
+  }
+}
 
 __device__ __forceinline__ f32x4_t mfma(const u32x4_t a, const u32x4_t b, f32x4_t c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
@@ -555,37 +581,41 @@ __device__ __forceinline__ void store_state0(const Consumer& C, const Wkv7Args& 
 
 }  // namespace
 
-// Barrier schedule (period k ends with barrier k; every wave executes nchunks + NPROD barriers):
-//   producer p works on chunk c = p + NPROD*m during periods c .. c+NPROD-1, one stage per period;
-//   consumers work on chunk c during period c + NPROD.
-// Slot c % RING is rewritten from period c on; its previous chunk c - RING was consumed in period c - 1.
-__global__ __launch_bounds__(512) void wkv7_chunk_fwd_kernel(Wkv7Args A) {
+// Slot c % RING holds chunk c.  Producer p fills it once every consumer has released chunk c - RING, then
+// publishes ready = c + 1; consumers take chunks in order.  Every wait is for a strictly earlier chunk, so the
+// hand-shake cannot cycle.
+__global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_fwd_kernel(Wkv7Args A) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   Slot* slots = reinterpret_cast<Slot*>(smem_raw);
   SnapSlot* snapslot = reinterpret_cast<SnapSlot*>(smem_raw + RING * sizeof(Slot));
+  Sync* sy = reinterpret_cast<Sync*>(smem_raw + RING * sizeof(Slot) + sizeof(SnapSlot));
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   const int64_t b = blockIdx.x / A.H, h = blockIdx.x % A.H;
   int64_t L = A.length ? (int64_t)A.length[b] : A.T;
   L = L < A.T ? L : A.T;
   const int64_t nchunks = (A.T + CK - 1) / CK;
+  if (threadIdx.x < sizeof(Sync) / sizeof(int)) reinterpret_cast<int*>(sy)[threadIdx.x] = 0;
+  __syncthreads();
 
-  if (wave < 4) {
+  if (wave < NCONS) {
     const bool q2drop = (A.flags & 1u) && L < A.T && A.ns != nullptr && A.ns[b * A.T + L] != 0;
     Consumer C;
     C.q = wave;
     C.lane = lane;
     load_state(C, A, b, h);
     if (L == 0) store_state0(C, A, b, h, q2drop);
-    for (int i = 0; i < NPROD; ++i) __syncthreads();
     for (int64_t c = 0; c < nchunks; ++c) {
       const int64_t c0 = c * CK;
       const int nvalid = (int)((A.T - c0 < CK) ? (A.T - c0) : CK);
-      consume(C, &slots[c % RING], snapslot, A, b, h, c0, nvalid, q2drop);
-      __syncthreads();
+      const int si = (int)(c % RING);
+      wait_ready(sy, si, (int)c + 1);
+      consume(C, &slots[si], snapslot, A, b, h, c0, nvalid, q2drop);
+      // every LDS read of the slot has returned (its data was used above)
+      if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], (int)c + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
   } else {
-    const int p = wave - 4;
+    const int p = wave - NCONS;
     Producer P;
     P.lane = lane;
     {
@@ -594,40 +624,36 @@ __global__ __launch_bounds__(512) void wkv7_chunk_fwd_kernel(Wkv7Args A) {
 #pragma unroll
       for (int x = 0; x < 2; ++x) {
         const int jj = 16 * x + n - 8 * g;
-        u32x4_t s = {0u, 0u, 0u, 0u};
-        if (jj >= 0 && jj < 8) s[jj >> 1] = (jj & 1) ? 0x3f800000u : 0x00003f80u;
-        P.sel[x] = s;
+        u32x4_t sl = {0u, 0u, 0u, 0u};
+        if (jj >= 0 && jj < 8) sl[jj >> 1] = (jj & 1) ? 0x3f800000u : 0x00003f80u;
+        P.sel[x] = sl;
       }
     }
-    for (int i = 0; i < p; ++i) __syncthreads();
-    int64_t done = p;
     Raw raw;
     if (p < nchunks) load_raw(raw, A, b, h, (int64_t)p * CK, lane);
     for (int64_t c = p; c < nchunks; c += NPROD) {
       const int64_t c0 = c * CK;
       const ChunkFlags F = chunk_flags(A, b, c0, L, lane);
-      Slot* slot = &slots[c % RING];
+      const int si = (int)(c % RING);
+      Slot* slot = &slots[si];
+      if (c >= RING) wait_consumed(sy, si, (int)(c - RING) + 1, lane);
       prod_stage0(P, raw, F, slot, snapslot);
-      __syncthreads();
+      if (c + NPROD < nchunks) load_raw(raw, A, b, h, c0 + NPROD * CK, lane);
       prod_stage1(P);
-      __syncthreads();
-      if (c + NPROD < nchunks) load_raw(raw, A, b, h, c0 + NPROD * CK, lane);   // needed two periods from now
       prod_stage2(P, F, slot);
-      __syncthreads();
       prod_stage3(P, F, slot, snapslot);
-      __syncthreads();
-      done += NPROD;
+      // the release orders this wave's LDS writes before the sequence number
+      if (lane == 0) __hip_atomic_store(&sy->ready[si], (int)c + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
-    for (int64_t i = done; i < nchunks + NPROD; ++i) __syncthreads();
   }
 }
 
 hipError_t launch_wkv7_chunk_fwd(const Wkv7Args& A, hipStream_t stream) {
-  const size_t smem = RING * sizeof(Slot) + sizeof(SnapSlot);
+  const size_t smem = RING * sizeof(Slot) + sizeof(SnapSlot) + sizeof(Sync);
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(wkv7_chunk_fwd_kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(wkv7_chunk_fwd_kernel, dim3((unsigned)(A.B * A.H)), dim3(512), smem, stream, A);
+  hipLaunchKernelGGL(wkv7_chunk_fwd_kernel, dim3((unsigned)(A.B * A.H)), dim3(64 * (NCONS + NPROD)), smem, stream, A);
   return hipGetLastError();
 }
 
