@@ -81,6 +81,24 @@ def cpu_baseline(sample_heads=2, threads=None):
                       f"(oracle.wkv7.wkv7_assoc_scan, NumPy/BLAS threads), {dt:.1f} s, scaled by heads"}
 
 
+def cpu_baseline_sequential(tokens=1024):
+    """Second CPU number: the oracle's sequential O(T N^2) recurrence (float64 NumPy), all 32 heads of one sequence."""
+    from oracle import wkv7 as o7
+    g = np.random.default_rng(2)
+    shp = (1, tokens, H, N)
+    r, k, v = (g.standard_normal(shp) for _ in range(3))
+    w = -0.5 + 0.5 * g.standard_normal(shp)
+    kap = g.standard_normal(shp)
+    kap /= np.linalg.norm(kap, axis=-1, keepdims=True)
+    a, b = -kap, kap / (1.0 + np.exp(-g.standard_normal(shp)))
+    s = 0.1 * g.standard_normal((1, H, N, N))
+    t0 = time.perf_counter()
+    o7.wkv7_base(r, w, k, v, a, b, s)
+    dt = time.perf_counter() - t0
+    return {"value": tokens / dt, "unit": "tokens/s", "cores": 1, "kind": "port",
+            "sample": f"1 sequence, T={tokens}, all {H} heads, float64 sequential loop (oracle.wkv7.wkv7_base), {dt:.1f} s"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -89,6 +107,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-bwd", action="store_true")
     ap.add_argument("--seq", action="store_true", help="force the sequential fp32 VALU kernel")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run three 1 GiB device copies before the timed region (scale for rocprofv3 --pmc)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the op shards over batch/heads "
@@ -103,9 +123,17 @@ def main():
     x = make_inputs(torch)
     tokens = B * T
 
+    if args.copy_probe:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     def fwd():
         return ops.wkv7_fwd(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], x["length"], x["new_starts"],
-                            compat=True, want_sa=False)
+                            compat=True, want_sa=False, force_seq=args.seq)
 
     wall, per_call = time_region(torch, fwd, args.steps, args.warmup)
     ms_step = 1e3 * wall / args.steps
@@ -139,6 +167,7 @@ def main():
                           "hbm_frac": fb_bytes / (ms2 * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": fb_bytes}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
+        out["cpu_baseline_sequential"] = cpu_baseline_sequential()
         out["gpu_over_cpu"] = out["value"] / out["cpu_baseline"]["value"]
     print(json.dumps(out))
 

@@ -47,21 +47,24 @@ constexpr int CK = 16;            // tokens per chunk
 constexpr int RS = 72;            // row stride (bf16 elements) of the [token][64] LDS arrays: 144 B (16-byte aligned rows)
 constexpr int NPROD = 4;          // producer waves; producer p owns chunks p, p + NPROD, ...
 constexpr int NCONS = 4;          // consumer waves, one per 16 value rows
-constexpr int RING = 6;           // slots in flight
+constexpr int RING = 5;           // slots in flight
 constexpr int SPIN_LIMIT = 1 << 16;   // polls before a waiter gives up (milliseconds; a healthy wait is microseconds)
 constexpr float LOG2E = 1.44269504088896340736f;
 constexpr float MIN_STEP_L2 = -1.0e4f;          // keeps the running sum finite
 constexpr float MIN_CUM_L2 = -80.0f * LOG2E;    // 2^MIN_CUM_L2 = e^-80
 
 // One chunk's operands as the consumers read them.  "lane-indexed" arrays hold, for every lane of the producer,
-// the 8 bytes that the same lane of a consumer loads: accumulator-layout registers (column lane%16, rows
-// 4*(lane/16)..+3) packed to bf16, which is exactly the A-operand layout (row lane%16, k-slots 4*(lane/16)..+3).
+// the 16 bytes that the same lane of a consumer loads: accumulator-layout registers (column lane%16, rows
+// 4*(lane/16)..+3) packed to bf16, hi pair then lo pair, which is exactly an A operand (row lane%16, k-slots
+// 4*(lane/16)..+3 of the hi part followed by the same slots of the lo part).
 struct __attribute__((aligned(16))) Slot {
-  uint16_t At[2][CK][RS];      // hi/lo of a_t.Ee_t; rows the entering state does not reach are zero
-  uint16_t Qt[2][CK][RS];      // hi/lo of r_t.E_t; same masking, plus rows whose y is defined as zero
-  uint2 BT[2][2][4][64];       // [bh|kh][hi|lo][key tile]: (b_s/E_s)^T, lane-indexed; masked for the chunk-end state
+  // At = a_t.Ee_t and Qt = r_t.E_t, [hi|lo][At|Qt][token][RS]: within a row, the 16-byte vector (j, g) at element
+  // 32j + 8g holds keys 32j+4g..+3 followed by keys 32j+16+4g..+3, the key order of the consumers' state tiles.
+  // Rows the entering state does not reach are zero; Qt rows whose y is defined as zero are zero.
+  uint16_t AQ[2][2][CK][RS];
+  uint4 BT[2][4][64];          // [bh|kh][key tile]: (b_s/E_s)^T hi,lo, lane-indexed; masked for the chunk-end state
   uint2 VT[4][64];             // v^T per value tile, lane-indexed
-  uint2 Mt[4][2][64];          // T, Mka, Mbr, Mkr: hi/lo, lane-indexed
+  uint4 Mt[4][64];             // T, Mka, Mbr, Mkr: hi,lo, lane-indexed
   float gamma[64];             // E at the chunk end
   int snap;                    // -1, or the in-chunk index of token length-1
   int keep_end;                // the entering state survives to the chunk end (no reset in the chunk)
@@ -70,7 +73,7 @@ struct __attribute__((aligned(16))) Slot {
 };
 // Update operands masked for the snapshot token; only one chunk per sequence needs them.
 struct __attribute__((aligned(16))) SnapSlot {
-  uint2 BT[2][2][4][64];
+  uint4 BT[2][4][64];
   float gamma[64];
 };
 // Hand-shake words.  ready[s] = c + 1 once chunk c is complete in slot s; consumed[q][s] = c + 1 once consumer
@@ -110,9 +113,16 @@ __device__ __forceinline__ uint32_t pack_exact(float x0, float x1) {
 
 // (x0, x1) -> packed truncated-bf16 hi parts and packed bf16 lo parts (x = hi + lo up to 2^-17 relative)
 __device__ __forceinline__ void split2(float x0, float x1, uint32_t& hi, uint32_t& lo) {
-  const uint32_t u0 = __float_as_uint(x0), u1 = __float_as_uint(x1);
-  hi = __builtin_amdgcn_perm(u1, u0, 0x07060302u);
-  lo = pack_rn(x0 - __uint_as_float(u0 & 0xffff0000u), x1 - __uint_as_float(u1 & 0xffff0000u));
+  hi = __builtin_amdgcn_perm(__float_as_uint(x1), __float_as_uint(x0), 0x07060302u);
+  // x - hi in one v_dot2c_f32_bf16 each: acc += hi.lo * -1 + hi.hi * 0  (resp. 0, -1)
+  // The two selectors are kept out of the compiler's sight: written as immediates, (-1, 0) would be encoded as
+  // the 16-bit inline constant -1.0, whose bit pattern is the fp16 one.
+  const bf16x2_t hp = __builtin_bit_cast(bf16x2_t, hi);
+  uint32_t m10 = 0x0000bf80u, m01 = 0xbf800000u;
+  asm volatile("" : "+s"(m10), "+s"(m01));
+  const float l0 = __builtin_amdgcn_fdot2_f32_bf16(hp, __builtin_bit_cast(bf16x2_t, m10), x0, false);
+  const float l1 = __builtin_amdgcn_fdot2_f32_bf16(hp, __builtin_bit_cast(bf16x2_t, m01), x1, false);
+  lo = pack_rn(l0, l1);
 }
 
 template <int CTRL>
@@ -166,129 +176,170 @@ __device__ __forceinline__ void load_raw(Raw& x, const Wkv7Args& A, int64_t b, i
   }
 }
 
-__device__ __forceinline__ void unpack16(const uint4 (&p)[2], float (&o)[16]) {
-  const uint32_t w[8] = {p[0].x, p[0].y, p[0].z, p[0].w, p[1].x, p[1].y, p[1].z, p[1].w};
+__device__ __forceinline__ void unpack8(const uint4 p, float (&o)[8]) {
+  const uint32_t w[4] = {p.x, p.y, p.z, p.w};
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
+  for (int i = 0; i < 4; ++i) {
     o[2 * i] = __uint_as_float(w[i] << 16);
     o[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
   }
 }
 
-// element e of a lane's 16 keys -> key index
-__device__ __forceinline__ int key_of(int g, int e) { return (e < 8) ? 8 * g + e : 32 + 8 * g + (e - 8); }
-
-// Producer state carried from one period to the next (registers).
 struct Producer {
   int lane;
   u32x4_t sel[2];     // B operands that pick keys 16*(tile%2)..+15 out of a 32-key half: MFMA as a transposer
-  // stage 0 -> 1
-  float pa[16], pq[16], pk[16], pb[16];   // a.Ee, r.E, k/E, b/E
-  // stage 1 -> 2,3
-  u32x4_t at_h[2], at_l[2], qt_h[2], qt_l[2], kh_h[2], kh_l[2], bh_h[2], bh_l[2];
-  f32x4_t Mba, MbaT, Mka, Mbr, Mkr;
 };
 
-// stage 0: decay scan and scaled operands (fp32); v^T and the chunk-end decay go straight to the slot
-__device__ __forceinline__ void prod_stage0(Producer& P, const Raw& x, const ChunkFlags& F, Slot* __restrict__ slot,
-                                            SnapSlot* __restrict__ snap) {
+// Everything of one chunk that does not depend on the entering state.  The two 32-key halves go through the
+// same pipeline one after the other (scan, scaling, hi/lo split, LDS parking, transposes, partial Gram sums),
+// which keeps the live register set small enough for three waves per SIMD.
+__device__ __forceinline__ void produce(const Producer& P, const Raw& x, const ChunkFlags& F, Slot* __restrict__ slot,
+                                        SnapSlot* __restrict__ snap) {
   const int lane = P.lane, t = lane & 15, g = lane >> 4;
   const bool valid = t < F.nvalid;
-  float fr[16], fk[16], fa[16], fb[16], E[16];
-  unpack16(x.r, fr); unpack16(x.k, fk); unpack16(x.a, fa); unpack16(x.b, fb);
-  {
-    // transpose by MFMA: D[token][value of tile] = sum_k V[token][k] sel[k][value]; the accumulator layout of D
-    // (lane = value, registers = 4 consecutive tokens) is the B-operand layout the consumers need
-    const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int tile = 0; tile < 4; ++tile) {
-      const uint4 vr = x.v[tile >> 1];
-      const u32x4_t vop = {vr.x, vr.y, vr.z, vr.w};
-      const f32x4_t dv = mfma(vop, P.sel[tile & 1], zero4);
-      slot->VT[tile][lane] = make_uint2(pack_exact(dv[0], dv[1]), pack_exact(dv[2], dv[3]));
-    }
-  }
-  {
-    float fw[16];
-    unpack16(x.w, fw);
-    // log2 of the decay, cumulative over the 16 tokens of the chunk (lanes of one DPP row)
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      float l2 = valid ? fmaxf(-exp2_fast(fw[e] * LOG2E) * LOG2E, MIN_STEP_L2) : 0.f;
-      l2 += dpp0<0x111>(l2);
-      l2 += dpp0<0x112>(l2);
-      l2 += dpp0<0x114>(l2);
-      l2 += dpp0<0x118>(l2);
-      E[e] = l2;
-    }
-  }
-  const bool slow = (F.ns & 0xffffu) != 0;
-  if (slow) {
-    // restart the cumulative decay at the last reset at or before this token
-    const uint32_t upto = F.ns & ((2u << t) - 1u) & 0xffffu;
-    const int p = upto ? 31 - __builtin_clz(upto) : 0;   // position of that reset
-    const int src = (lane & 48) | (p > 0 ? p - 1 : 0);
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const float base = __shfl(E[e], src, 64);
-      if (p > 0) E[e] -= base;
-    }
-    if ((F.ns >> t) & 1u) {
-#pragma unroll
-      for (int e = 0; e < 16; ++e) fa[e] = 0.f;   // the state entering a reset token is zero: sa = 0
-    }
-  }
-#pragma unroll
-  for (int e = 0; e < 16; ++e) {
-    const float l2 = fmaxf(E[e], MIN_CUM_L2);
-    const float Ev = exp2_fast(l2), Einv = exp2_fast(-l2);
-    // exclusive: value of the previous token; 1 for the first token of the chunk
-    const float Ee = __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(1.0f), __float_as_int(Ev), 0x111, 0xf, 0xf, false));
-    P.pa[e] = fa[e] * Ee;      // at a reset token a is zero, whatever Ee holds
-    P.pq[e] = fr[e] * Ev;
-    P.pk[e] = fk[e] * Einv;
-    P.pb[e] = fb[e] * Einv;
-    E[e] = Ev;
-  }
-  if (t == 15) {
-#pragma unroll
-    for (int hf = 0; hf < 2; ++hf) {
-      float* gp = &slot->gamma[8 * g + 32 * hf];
-      *reinterpret_cast<float4*>(gp) = make_float4(E[8 * hf], E[8 * hf + 1], E[8 * hf + 2], E[8 * hf + 3]);
-      *reinterpret_cast<float4*>(gp + 4) = make_float4(E[8 * hf + 4], E[8 * hf + 5], E[8 * hf + 6], E[8 * hf + 7]);
-    }
-  }
-  if (t == F.snap) {
-#pragma unroll
-    for (int e = 0; e < 16; ++e) snap->gamma[key_of(g, e)] = E[e];
-  }
-}
-
-// stage 1: hi/lo split and the five Gram tiles
-__device__ __forceinline__ void prod_stage1(Producer& P) {
-#pragma unroll
-  for (int hf = 0; hf < 2; ++hf) {
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int e = 8 * hf + 2 * j;
-      uint32_t hi, lo;
-      split2(P.pa[e], P.pa[e + 1], hi, lo); P.at_h[hf][j] = hi; P.at_l[hf][j] = lo;
-      split2(P.pq[e], P.pq[e + 1], hi, lo); P.qt_h[hf][j] = hi; P.qt_l[hf][j] = lo;
-      split2(P.pk[e], P.pk[e + 1], hi, lo); P.kh_h[hf][j] = hi; P.kh_l[hf][j] = lo;
-      split2(P.pb[e], P.pb[e + 1], hi, lo); P.bh_h[hf][j] = hi; P.bh_l[hf][j] = lo;
-    }
-  }
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+  const u32x4_t z4 = {0u, 0u, 0u, 0u};
+  const bool slow = F.ns != 0;                    // a reset in this chunk or at the first token of the next
+  const uint32_t resets = F.ns & 0xffffu;
+  // reset bookkeeping (uniform values unless they depend on t)
+  int lastseg = 0, seg_src = 0;
+  bool s0_reaches = true, q_keep = true, restart = false, at_reset = false;
+  uint32_t keep_upd = 0xffffu, keep_snap = 0;
+  if (F.snap >= 0) keep_snap = (2u << F.snap) - 1u;
+  if (slow) {
+    lastseg = seg_of(F.ns, 15);
+    s0_reaches = seg_of(F.ns, t) == 0;                              // the entering state reaches this token
+    q_keep = s0_reaches && !(F.compat && ((F.ns >> (t + 1)) & 1u)); // y[t] is defined as zero before a reset
+    if (resets) keep_upd = 0xffffu & ~((1u << (31 - __builtin_clz(resets))) - 1u);   // tokens from the last reset on
+    const uint32_t upto = resets & ((2u << t) - 1u);
+    const int pr = upto ? 31 - __builtin_clz(upto) : 0;             // last reset at or before this token
+    restart = pr > 0;
+    seg_src = (lane & 48) | (pr > 0 ? pr - 1 : 0);
+    at_reset = (resets >> t) & 1u;
+    if (F.snap >= 0) {
+      const uint32_t us = resets & keep_snap;
+      if (us) keep_snap &= ~((1u << (31 - __builtin_clz(us))) - 1u);
+    }
+  }
+  auto masked_pack = [&](const f32x4_t d, uint32_t keep) {
+    const uint32_t bits = keep >> (4 * g);
+    const float d0 = (bits & 1u) ? d[0] : 0.f, d1 = (bits & 2u) ? d[1] : 0.f;
+    const float d2 = (bits & 4u) ? d[2] : 0.f, d3 = (bits & 8u) ? d[3] : 0.f;
+    return make_uint2(pack_exact(d0, d1), pack_exact(d2, d3));
+  };
+  auto plain_pack = [&](const f32x4_t d) { return make_uint2(pack_exact(d[0], d[1]), pack_exact(d[2], d[3])); };
+  auto join = [&](const uint2 hi, const uint2 lo) { return make_uint4(hi.x, hi.y, lo.x, lo.y); };
+
   f32x4_t Mba = zero4, MbaT = zero4, Mka = zero4, Mbr = zero4, Mkr = zero4;
-  // accumulator layout: lane holds column n = lane%16, rows m = 4g..4g+3.  Five independent chains, interleaved.
 #pragma unroll
   for (int hf = 0; hf < 2; ++hf) {
+    // ---- v^T of value tiles 2hf, 2hf+1: D[token][value] = sum_k V[token][k] sel[k][value]
+    {
+      const uint4 vr = x.v[hf];
+      const u32x4_t vop = {vr.x, vr.y, vr.z, vr.w};
+#pragma unroll
+      for (int x2 = 0; x2 < 2; ++x2) slot->VT[2 * hf + x2][lane] = plain_pack(mfma(vop, P.sel[x2], zero4));
+    }
+    // ---- decay scan over the 16 tokens (lanes of one DPP row), log2 domain
+    float E[8], fa[8];
+    {
+      float fw[8];
+      unpack8(x.w[hf], fw);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        float l2 = fmaxf(-exp2_fast(fw[e] * LOG2E) * LOG2E, MIN_STEP_L2);
+        if (F.nvalid != CK) l2 = valid ? l2 : 0.f;
+        l2 += dpp0<0x111>(l2);
+        l2 += dpp0<0x112>(l2);
+        l2 += dpp0<0x114>(l2);
+        l2 += dpp0<0x118>(l2);
+        E[e] = l2;
+      }
+    }
+    unpack8(x.a[hf], fa);
+    if (slow) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float base = __shfl(E[e], seg_src, 64);   // restart the cumulative decay at the last reset
+        if (restart) E[e] -= base;
+        if (at_reset) fa[e] = 0.f;                      // the state entering a reset token is zero: sa = 0
+      }
+    }
+    // ---- scaled operands and their hi/lo split
+    u32x4_t at_h, at_l, qt_h, qt_l, kh_h, kh_l, bh_h, bh_l;
+    {
+      float fr[8], fk[8], fb[8], Einv[8], Ee[8];
+      unpack8(x.r[hf], fr); unpack8(x.k[hf], fk); unpack8(x.b[hf], fb);
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float l2 = fmaxf(E[e], MIN_CUM_L2);
+        E[e] = exp2_fast(l2);
+        Einv[e] = exp2_fast(-l2);
+        // exclusive: value of the previous token; 1 for the first token of the chunk (a is zero at reset tokens)
+        Ee[e] = __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(1.0f), __float_as_int(E[e]), 0x111, 0xf, 0xf, false));
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int e = 2 * j;
+        uint32_t hi, lo;
+        split2(fa[e] * Ee[e], fa[e + 1] * Ee[e + 1], hi, lo); at_h[j] = hi; at_l[j] = lo;
+        split2(fr[e] * E[e], fr[e + 1] * E[e + 1], hi, lo); qt_h[j] = hi; qt_l[j] = lo;
+        split2(fk[e] * Einv[e], fk[e + 1] * Einv[e + 1], hi, lo); kh_h[j] = hi; kh_l[j] = lo;
+        split2(fb[e] * Einv[e], fb[e + 1] * Einv[e + 1], hi, lo); bh_h[j] = hi; bh_l[j] = lo;
+      }
+    }
+    // ---- decay to the chunk end / to the snapshot token
+    if (t == 15) {
+      float* gp = &slot->gamma[8 * g + 32 * hf];
+      *reinterpret_cast<float4*>(gp) = make_float4(E[0], E[1], E[2], E[3]);
+      *reinterpret_cast<float4*>(gp + 4) = make_float4(E[4], E[5], E[6], E[7]);
+    }
+    if (t == F.snap) {
+      float* gp = &snap->gamma[8 * g + 32 * hf];
+      *reinterpret_cast<float4*>(gp) = make_float4(E[0], E[1], E[2], E[3]);
+      *reinterpret_cast<float4*>(gp + 4) = make_float4(E[4], E[5], E[6], E[7]);
+    }
+    // ---- At, Qt rows for the consumers, in their key order: this lane's keys 8g..8g+3 and 8g+4..8g+7 of the half
+    //      are the (g>>1)-th 8-byte piece of the vectors 2(g&1) and 2(g&1)+1 of block j = hf
+    {
+      const int e0 = 32 * hf + 16 * (g & 1) + 4 * (g >> 1);     // element offset of the first piece
+      auto put = [&](uint16_t* row, const u32x4_t v, bool keep) {
+        *reinterpret_cast<uint2*>(row + e0) = keep ? make_uint2(v[0], v[1]) : make_uint2(0u, 0u);
+        *reinterpret_cast<uint2*>(row + e0 + 8) = keep ? make_uint2(v[2], v[3]) : make_uint2(0u, 0u);
+      };
+      if (!slow) {
+        put(slot->AQ[0][0][t], at_h, true); put(slot->AQ[1][0][t], at_l, true);
+        put(slot->AQ[0][1][t], qt_h, true); put(slot->AQ[1][1][t], qt_l, true);
+      } else {
+        put(slot->AQ[0][0][t], at_h, s0_reaches); put(slot->AQ[1][0][t], at_l, s0_reaches);
+        put(slot->AQ[0][1][t], qt_h, q_keep); put(slot->AQ[1][1][t], qt_l, q_keep);
+      }
+    }
+    // ---- (b/E)^T, (k/E)^T of key tiles 2hf, 2hf+1 by MFMA: the accumulator layout of D (lane = key, registers =
+    //      4 consecutive tokens) is the A-operand layout of the state update
+#pragma unroll
+    for (int x2 = 0; x2 < 2; ++x2) {
+      const int tile = 2 * hf + x2;
+      const u32x4_t sel = P.sel[x2];
+      const f32x4_t dbh = mfma(bh_h, sel, zero4), dbl = mfma(bh_l, sel, zero4);
+      const f32x4_t dkh = mfma(kh_h, sel, zero4), dkl = mfma(kh_l, sel, zero4);
+      if (keep_upd == 0xffffu) {
+        slot->BT[0][tile][lane] = join(plain_pack(dbh), plain_pack(dbl));
+        slot->BT[1][tile][lane] = join(plain_pack(dkh), plain_pack(dkl));
+      } else {
+        slot->BT[0][tile][lane] = join(masked_pack(dbh, keep_upd), masked_pack(dbl, keep_upd));
+        slot->BT[1][tile][lane] = join(masked_pack(dkh, keep_upd), masked_pack(dkl, keep_upd));
+      }
+      if (F.snap >= 0) {
+        snap->BT[0][tile][lane] = join(masked_pack(dbh, keep_snap), masked_pack(dbl, keep_snap));
+        snap->BT[1][tile][lane] = join(masked_pack(dkh, keep_snap), masked_pack(dkl, keep_snap));
+      }
+    }
+    // ---- partial Gram sums over this half's keys (accumulator layout: column n = lane%16, rows 4g..4g+3)
 #pragma unroll
     for (int part = 0; part < 3; ++part) {
-      const u32x4_t bA = part == 2 ? P.bh_l[hf] : P.bh_h[hf], kA = part == 2 ? P.kh_l[hf] : P.kh_h[hf];
-      const u32x4_t aA = part == 2 ? P.at_l[hf] : P.at_h[hf];
-      const u32x4_t aB = part == 1 ? P.at_l[hf] : P.at_h[hf], qB = part == 1 ? P.qt_l[hf] : P.qt_h[hf];
-      const u32x4_t bB = part == 1 ? P.bh_l[hf] : P.bh_h[hf];
+      const u32x4_t bA = part == 2 ? bh_l : bh_h, kA = part == 2 ? kh_l : kh_h, aA = part == 2 ? at_l : at_h;
+      const u32x4_t aB = part == 1 ? at_l : at_h, qB = part == 1 ? qt_l : qt_h, bB = part == 1 ? bh_l : bh_h;
       Mba = mfma(bA, aB, Mba);     // [s][t] = bh_s . at_t
       MbaT = mfma(aA, bB, MbaT);   // [t][s]
       Mka = mfma(kA, aB, Mka);     // [s][t] = kh_s . at_t
@@ -296,15 +347,8 @@ __device__ __forceinline__ void prod_stage1(Producer& P) {
       Mkr = mfma(kA, qB, Mkr);     // [s][t] = kh_s . qt_t
     }
   }
-  P.Mba = Mba; P.MbaT = MbaT; P.Mka = Mka; P.Mbr = Mbr; P.Mkr = Mkr;
-}
-
-// stage 2: triangular masks, T = (I - Mba)^{-1}, park T / Mka / Mbr / Mkr
-__device__ __forceinline__ void prod_stage2(Producer& P, const ChunkFlags& F, Slot* __restrict__ slot) {
-  const int lane = P.lane, n = lane & 15, g = lane >> 4;
-  const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
-  f32x4_t Mba = P.Mba, MbaT = P.MbaT, Mka = P.Mka, Mbr = P.Mbr, Mkr = P.Mkr;
-  const bool slow = F.ns != 0;
+  // ---- triangular masks
+  const int n = t;
   if (!slow) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -329,7 +373,7 @@ __device__ __forceinline__ void prod_stage2(Producer& P, const ChunkFlags& F, Sl
       MbaT[i] = gt ? MbaT[i] : 0.f;
     }
   }
-  // T = (I + M^8)(I + M^4)(I + M^2)(I + M), single-bf16 operands
+  // ---- T = (I + M^8)(I + M^4)(I + M^2)(I + M), single-bf16 operands
   auto single = [&](const f32x4_t d) {
     u32x4_t o = {pack_rn(d[0], d[1]), pack_rn(d[2], d[3]), 0u, 0u};
     return o;
@@ -350,78 +394,9 @@ __device__ __forceinline__ void prod_stage2(Producer& P, const ChunkFlags& F, Sl
   auto park = [&](int which, const f32x4_t d) {
     split2(d[0], d[1], hi0, lo0);
     split2(d[2], d[3], hi1, lo1);
-    slot->Mt[which][0][lane] = make_uint2(hi0, hi1);
-    slot->Mt[which][1][lane] = make_uint2(lo0, lo1);
+    slot->Mt[which][lane] = make_uint4(hi0, hi1, lo0, lo1);
   };
   park(0, Pm); park(1, Mka); park(2, Mbr); park(3, Mkr);
-}
-
-// stage 3: operands the consumers read through LDS: At, Qt (row-major), transposed bh / kh, flags
-__device__ __forceinline__ void prod_stage3(Producer& P, const ChunkFlags& F, Slot* __restrict__ slot,
-                                            SnapSlot* __restrict__ snap) {
-  const int lane = P.lane, t = lane & 15, g = lane >> 4;
-  const bool slow = F.ns != 0;
-  const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
-  const u32x4_t z4 = {0u, 0u, 0u, 0u};
-  int lastseg = 0;
-  bool s0_reaches = true, q_keep = true;
-  uint32_t keep_upd = 0xffffu;       // tokens that still contribute to the chunk-end state
-  if (slow) {
-    lastseg = seg_of(F.ns, 15);
-    s0_reaches = seg_of(F.ns, t) == 0;                             // the entering state reaches this token
-    q_keep = s0_reaches && !(F.compat && ((F.ns >> (t + 1)) & 1u));
-    const uint32_t resets = F.ns & 0xffffu;
-    // tokens from the last reset on
-    keep_upd = resets ? (0xffffu & ~((1u << (31 - __builtin_clz(resets))) - 1u)) : 0xffffu;
-  }
-#pragma unroll
-  for (int hf = 0; hf < 2; ++hf) {
-    const int col = 8 * g + 32 * hf;
-    *reinterpret_cast<u32x4_t*>(&slot->At[0][t][col]) = s0_reaches ? P.at_h[hf] : z4;
-    *reinterpret_cast<u32x4_t*>(&slot->At[1][t][col]) = s0_reaches ? P.at_l[hf] : z4;
-    *reinterpret_cast<u32x4_t*>(&slot->Qt[0][t][col]) = q_keep ? P.qt_h[hf] : z4;
-    *reinterpret_cast<u32x4_t*>(&slot->Qt[1][t][col]) = q_keep ? P.qt_l[hf] : z4;
-  }
-  // transposes by MFMA: D[token][key of tile] = sum_k X[token][k] sel[k][key]; the accumulator layout of D
-  // (lane = key, registers = 4 consecutive tokens) is the A-operand layout of the state update
-  uint32_t keep_snap = 0;
-  if (F.snap >= 0) {
-    keep_snap = (2u << F.snap) - 1u;
-    if (slow) {
-      const uint32_t upto = F.ns & keep_snap & 0xffffu;
-      if (upto) keep_snap &= ~((1u << (31 - __builtin_clz(upto))) - 1u);
-    }
-  }
-  auto masked_pack = [&](const f32x4_t d, uint32_t keep) {
-    const uint32_t bits = keep >> (4 * g);
-    const float d0 = (bits & 1u) ? d[0] : 0.f, d1 = (bits & 2u) ? d[1] : 0.f;
-    const float d2 = (bits & 4u) ? d[2] : 0.f, d3 = (bits & 8u) ? d[3] : 0.f;
-    return make_uint2(pack_exact(d0, d1), pack_exact(d2, d3));
-  };
-#pragma unroll
-  for (int tile = 0; tile < 4; ++tile) {
-    const int hf = tile >> 1;
-    const u32x4_t sel = P.sel[tile & 1];
-    const f32x4_t dbh = mfma(P.bh_h[hf], sel, zero4), dbl = mfma(P.bh_l[hf], sel, zero4);
-    const f32x4_t dkh = mfma(P.kh_h[hf], sel, zero4), dkl = mfma(P.kh_l[hf], sel, zero4);
-    if (keep_upd == 0xffffu) {
-      slot->BT[0][0][tile][lane] = make_uint2(pack_exact(dbh[0], dbh[1]), pack_exact(dbh[2], dbh[3]));
-      slot->BT[0][1][tile][lane] = make_uint2(pack_exact(dbl[0], dbl[1]), pack_exact(dbl[2], dbl[3]));
-      slot->BT[1][0][tile][lane] = make_uint2(pack_exact(dkh[0], dkh[1]), pack_exact(dkh[2], dkh[3]));
-      slot->BT[1][1][tile][lane] = make_uint2(pack_exact(dkl[0], dkl[1]), pack_exact(dkl[2], dkl[3]));
-    } else {
-      slot->BT[0][0][tile][lane] = masked_pack(dbh, keep_upd);
-      slot->BT[0][1][tile][lane] = masked_pack(dbl, keep_upd);
-      slot->BT[1][0][tile][lane] = masked_pack(dkh, keep_upd);
-      slot->BT[1][1][tile][lane] = masked_pack(dkl, keep_upd);
-    }
-    if (F.snap >= 0) {
-      snap->BT[0][0][tile][lane] = masked_pack(dbh, keep_snap);
-      snap->BT[0][1][tile][lane] = masked_pack(dbl, keep_snap);
-      snap->BT[1][0][tile][lane] = masked_pack(dkh, keep_snap);
-      snap->BT[1][1][tile][lane] = masked_pack(dkl, keep_snap);
-    }
-  }
   if (lane == 0) {
     slot->snap = F.snap;
     slot->keep_end = (lastseg == 0) ? 1 : 0;
@@ -437,12 +412,58 @@ struct Consumer {
   int q, lane;
 };
 
-__device__ __forceinline__ uint2 lds8(const uint16_t* p) { return *reinterpret_cast<const uint2*>(p); }
+// Operands a consumer needs at the start of a chunk; they are fetched from the slot while the previous chunk
+// is still being finished, so that their LDS latency is off the chunk-to-chunk dependency chain.
+struct Ops {
+  u32x4_t aq[2][2][2];     // [hi|lo][At|Qt][j]: rows in the key order of the state tiles
+  u32x4_t T, Ka, Br, Kr;   // T, Mka, Mbr, Mkr: hi pair, lo pair
+  u32x4_t vv;              // v^T of this wave's value tile, twice (for a hi and a lo A part side by side)
+  int keep_end;
+};
 
-__device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ slot, const SnapSlot* __restrict__ snapslot,
-                                        const Wkv7Args& A, int64_t b, int64_t h, int64_t c0, int nvalid, bool q2drop) {
+__device__ __forceinline__ void load_ops(Ops& o, const Slot* __restrict__ slot, int q, int lane) {
+  const int n = lane & 15, g = lane >> 4;
+#pragma unroll
+  for (int pl = 0; pl < 2; ++pl)
+#pragma unroll
+    for (int ar = 0; ar < 2; ++ar)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        o.aq[pl][ar][j] = *reinterpret_cast<const u32x4_t*>(&slot->AQ[pl][ar][n][32 * j + 8 * g]);
+  o.T = *reinterpret_cast<const u32x4_t*>(&slot->Mt[0][lane]);
+  o.Ka = *reinterpret_cast<const u32x4_t*>(&slot->Mt[1][lane]);
+  o.Br = *reinterpret_cast<const u32x4_t*>(&slot->Mt[2][lane]);
+  o.Kr = *reinterpret_cast<const u32x4_t*>(&slot->Mt[3][lane]);
+  const uint2 v0 = slot->VT[q][lane], v1 = slot->VT[q][lane];
+  o.vv = u32x4_t{v0.x, v0.y, v1.x, v1.y};
+  o.keep_end = slot->keep_end;
+}
+
+// Uniform output cursors of a consumer, advanced by one chunk per call.
+struct OutCursor {
+  char* y;             // A.out at (b, c0, h, 0)
+  char* sa;            // A.sa at the same place, or null
+  size_t tok_bytes;    // bytes between consecutive tokens in y (twice that in sa)
+  uint32_t voff;       // lane part of the address, in elements: (4g * H) * 64 + value
+};
+
+// The S0-dependent part of one chunk.  `prefetch` runs once the update MFMAs are in flight: the caller uses it
+// to wait for, and fetch, the next chunk's operands.
+template <class Prefetch>
+__device__ __forceinline__ void consume(Consumer& C, const Ops& o, const Slot* __restrict__ slot,
+                                        const SnapSlot* __restrict__ snapslot, const Wkv7Args& A, int64_t b, int64_t h,
+                                        int nvalid, bool is_snap, bool q2drop, OutCursor& oc, Prefetch&& prefetch) {
   const int lane = C.lane, n = lane & 15, g = lane >> 4;
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+  // update operands of this chunk: needed last, so their latency hides behind the W / SA chain
+  u32x4_t bt[2][4];
+  float4 gm[4];
+#pragma unroll
+  for (int tile = 0; tile < 4; ++tile) {
+    bt[0][tile] = *reinterpret_cast<const u32x4_t*>(&slot->BT[0][tile][lane]);
+    bt[1][tile] = *reinterpret_cast<const u32x4_t*>(&slot->BT[1][tile][lane]);
+    gm[tile] = *reinterpret_cast<const float4*>(&slot->gamma[16 * tile + 4 * g]);
+  }
   // B operands from the state: MFMA j contracts over the keys of tiles 2j and 2j+1
   u32x4_t Sh[2], Sl[2];
 #pragma unroll
@@ -453,99 +474,94 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
     split2(C.S[2 * j + 1][0], C.S[2 * j + 1][1], hi, lo); Sh[j][2] = hi; Sl[j][2] = lo;
     split2(C.S[2 * j + 1][2], C.S[2 * j + 1][3], hi, lo); Sh[j][3] = hi; Sl[j][3] = lo;
   }
-  // A operands: rows = tokens (lane%16), same key order as the B operands above
-  auto rows = [&](const uint16_t (*arr)[RS], int j) {
-    const uint2 p0 = lds8(&arr[n][32 * j + 4 * g]);
-    const uint2 p1 = lds8(&arr[n][32 * j + 16 + 4 * g]);
-    u32x4_t o = {p0.x, p0.y, p1.x, p1.y};
-    return o;
-  };
-  f32x4_t W = zero4, Y = zero4;   // [token 4g+i][value n]
+  f32x4_t W = zero4, Y = zero4;   // [token 4g+i][value n], two interleaved accumulation chains
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
-    const u32x4_t ah = rows(slot->At[0], j), al = rows(slot->At[1], j);
-    const u32x4_t qh = rows(slot->Qt[0], j), ql = rows(slot->Qt[1], j);
-    W = mfma(ah, Sh[j], W);
-    Y = mfma(qh, Sh[j], Y);
-    W = mfma(ah, Sl[j], W);
-    Y = mfma(qh, Sl[j], Y);
-    W = mfma(al, Sh[j], W);
-    Y = mfma(ql, Sh[j], Y);
+    W = mfma(o.aq[0][0][j], Sh[j], W); Y = mfma(o.aq[0][1][j], Sh[j], Y);
+    W = mfma(o.aq[0][0][j], Sl[j], W); Y = mfma(o.aq[0][1][j], Sl[j], Y);
+    W = mfma(o.aq[1][0][j], Sh[j], W); Y = mfma(o.aq[1][1][j], Sh[j], Y);
   }
-  // v of the four tokens 4g..4g+3 for this lane's value column
-  const int val = 16 * C.q + n;
-  const uint2 vt = slot->VT[C.q][lane];
-  const uint32_t v01 = vt.x, v23 = vt.y;
-  const uint2 Th = slot->Mt[0][0][lane], Tl = slot->Mt[0][1][lane];
-  const uint2 Kah = slot->Mt[1][0][lane], Kal = slot->Mt[1][1][lane];
-  const uint2 Brh = slot->Mt[2][0][lane], Brl = slot->Mt[2][1][lane];
-  const uint2 Krh = slot->Mt[3][0][lane], Krl = slot->Mt[3][1][lane];
-  {
-    const u32x4_t a = {Kah.x, Kah.y, Kal.x, Kal.y}, bb = {v01, v23, v01, v23};
-    W = mfma(a, bb, W);                       // W += Mka^T V^T
-  }
-  uint32_t Wh0, Wl0, Wh1, Wl1;
-  split2(W[0], W[1], Wh0, Wl0);
-  split2(W[2], W[3], Wh1, Wl1);
+  W = mfma(o.Ka, o.vv, W);                    // W += Mka^T V^T (hi and lo parts side by side)
+  Y = mfma(o.Kr, o.vv, Y);                    // Y += Mkr^T V^T
+  uint32_t h0, l0, h1, l1;
+  split2(W[0], W[1], h0, l0);
+  split2(W[2], W[3], h1, l1);
   f32x4_t SA;
   {
-    const u32x4_t a1 = {Th.x, Th.y, Tl.x, Tl.y}, b1 = {Wh0, Wh1, Wh0, Wh1};
-    const u32x4_t a2 = {Th.x, Th.y, 0u, 0u}, b2 = {Wl0, Wl1, 0u, 0u};
-    SA = mfma(a1, b1, zero4);
-    SA = mfma(a2, b2, SA);                    // SA^T = T^T W^T
+    // an A operand holds the hi pair in k-slots 0..3 and the lo pair in 4..7: against (x_hi, x_hi) it gives
+    // (A_hi + A_lo) x_hi, against (x_lo, 0) it gives A_hi x_lo
+    const u32x4_t bhh = {h0, h1, h0, h1}, bl0 = {l0, l1, 0u, 0u};
+    SA = mfma(o.T, bhh, zero4);               // (T_hi + T_lo)^T W_hi
+    SA = mfma(o.T, bl0, SA);                  // T_hi^T W_lo
   }
-  uint32_t Ah0, Al0, Ah1, Al1;
-  split2(SA[0], SA[1], Ah0, Al0);
-  split2(SA[2], SA[3], Ah1, Al1);
-  const u32x4_t bSS = {Ah0, Ah1, Ah0, Ah1}, bLV = {Al0, Al1, v01, v23}, bV0 = {v01, v23, 0u, 0u};
-  {
-    const u32x4_t a1 = {Brh.x, Brh.y, Brl.x, Brl.y}, a2 = {Brh.x, Brh.y, Krh.x, Krh.y}, a3 = {Krl.x, Krl.y, 0u, 0u};
-    Y = mfma(a1, bSS, Y);
-    Y = mfma(a2, bLV, Y);
-    Y = mfma(a3, bV0, Y);                     // Y^T += Mbr^T SA^T + Mkr^T V^T
-  }
-  // state update (and the snapshot for `length`), tile by tile: rows = keys
-  auto update = [&](const uint2 (*bt)[2][4][64], const float* gam, bool keep, f32x4_t (&out)[4]) {
+  split2(SA[0], SA[1], h0, l0);
+  split2(SA[2], SA[3], h1, l1);
+  const u32x4_t sHH = {h0, h1, h0, h1}, sL0 = {l0, l1, 0u, 0u};
+  Y = mfma(o.Br, sHH, Y);
+  Y = mfma(o.Br, sL0, Y);                     // Y^T += Mbr^T SA^T
+  // state snapshot for `length` (one chunk per sequence)
+  if (is_snap) {
+    const bool keep = slot->keep_snap != 0;
 #pragma unroll
     for (int tile = 0; tile < 4; ++tile) {
-      const uint2 bh = bt[0][0][tile][lane], bl = bt[0][1][tile][lane];
-      const uint2 kh = bt[1][0][tile][lane], kl = bt[1][1][tile][lane];
-      const u32x4_t a1 = {bh.x, bh.y, bl.x, bl.y}, a2 = {bh.x, bh.y, kh.x, kh.y}, a3 = {kl.x, kl.y, 0u, 0u};
+      const u32x4_t sb = *reinterpret_cast<const u32x4_t*>(&snapslot->BT[0][tile][lane]);
+      const u32x4_t sk = *reinterpret_cast<const u32x4_t*>(&snapslot->BT[1][tile][lane]);
       f32x4_t acc = keep ? C.S[tile] : zero4;
-      acc = mfma(a1, bSS, acc);
-      acc = mfma(a2, bLV, acc);
-      acc = mfma(a3, bV0, acc);
-      const float4 gm = *reinterpret_cast<const float4*>(&gam[16 * tile + 4 * g]);
-      acc[0] *= gm.x; acc[1] *= gm.y; acc[2] *= gm.z; acc[3] *= gm.w;
-      out[tile] = acc;
-    }
-  };
-  if (slot->snap >= 0) {
-    f32x4_t snap[4];
-    update(snapslot->BT, snapslot->gamma, slot->keep_snap != 0, snap);
-#pragma unroll
-    for (int tile = 0; tile < 4; ++tile) {
-      const size_t off = (((size_t)b * A.H + h) * 64 + val) * 64 + 16 * tile + 4 * g;
+      acc = mfma(sb, sHH, acc);
+      acc = mfma(sk, o.vv, acc);
+      acc = mfma(sb, sL0, acc);
+      const float4 sg = *reinterpret_cast<const float4*>(&snapslot->gamma[16 * tile + 4 * g]);
+      acc[0] *= sg.x; acc[1] *= sg.y; acc[2] *= sg.z; acc[3] *= sg.w;
+      const size_t off = (((size_t)b * A.H + h) * 64 + 16 * C.q + n) * 64 + 16 * tile + 4 * g;
       if (A.st_f32) {
-        float4 o = q2drop ? make_float4(0.f, 0.f, 0.f, 0.f) : make_float4(snap[tile][0], snap[tile][1], snap[tile][2], snap[tile][3]);
-        *reinterpret_cast<float4*>(reinterpret_cast<float*>(A.new_s) + off) = o;
+        float4 ov = q2drop ? make_float4(0.f, 0.f, 0.f, 0.f) : make_float4(acc[0], acc[1], acc[2], acc[3]);
+        *reinterpret_cast<float4*>(reinterpret_cast<float*>(A.new_s) + off) = ov;
       } else {
-        uint2 o = q2drop ? make_uint2(0u, 0u) : make_uint2(pack_rn(snap[tile][0], snap[tile][1]), pack_rn(snap[tile][2], snap[tile][3]));
-        *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(A.new_s) + off) = o;
+        uint2 ov = q2drop ? make_uint2(0u, 0u) : make_uint2(pack_rn(acc[0], acc[1]), pack_rn(acc[2], acc[3]));
+        *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(A.new_s) + off) = ov;
       }
     }
   }
-  update(slot->BT, slot->gamma, slot->keep_end != 0, C.S);
-  // outputs: register i is token 4g+i, lanes n = 16 consecutive values
+  // state update, tile by tile: rows = keys.  S <- (S + Bh^T SA^T + Kh^T V^T) . gamma
+  if (!o.keep_end) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int tt = 4 * g + i;
-    if (tt < nvalid) {
-      const size_t off = (((size_t)b * A.T + c0 + tt) * A.H + h) * 64 + val;
-      reinterpret_cast<uint16_t*>(A.out)[off] = f32_to_bf16(Y[i]);
-      if (A.sa != nullptr) A.sa[off] = SA[i];
+    for (int tile = 0; tile < 4; ++tile) C.S[tile] = zero4;   // a reset inside the chunk cuts the entering state off
+  }
+#pragma unroll
+  for (int tile = 0; tile < 4; ++tile) {
+    f32x4_t acc = C.S[tile];
+    acc = mfma(bt[0][tile], sHH, acc);
+    acc = mfma(bt[1][tile], o.vv, acc);
+    acc = mfma(bt[0][tile], sL0, acc);
+    acc[0] *= gm[tile].x; acc[1] *= gm[tile].y; acc[2] *= gm[tile].z; acc[3] *= gm[tile].w;
+    C.S[tile] = acc;
+  }
+  prefetch();
+  // outputs: register i is token 4g+i, lanes n = 16 consecutive values
+  const uint32_t y01 = pack_rn(Y[0], Y[1]), y23 = pack_rn(Y[2], Y[3]);
+  char* const yl = oc.y + (size_t)oc.voff * 2;
+  if (nvalid == CK) {
+    *reinterpret_cast<uint16_t*>(yl) = (uint16_t)(y01 & 0xffffu);
+    *reinterpret_cast<uint16_t*>(yl + oc.tok_bytes) = (uint16_t)(y01 >> 16);
+    *reinterpret_cast<uint16_t*>(yl + 2 * oc.tok_bytes) = (uint16_t)(y23 & 0xffffu);
+    *reinterpret_cast<uint16_t*>(yl + 3 * oc.tok_bytes) = (uint16_t)(y23 >> 16);
+    if (oc.sa != nullptr) {
+      char* const sl = oc.sa + (size_t)oc.voff * 4;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) *reinterpret_cast<float*>(sl + 2 * i * oc.tok_bytes) = SA[i];
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (4 * g + i < nvalid) {
+        const uint32_t yv = (i & 2) ? y23 : y01;
+        *reinterpret_cast<uint16_t*>(yl + i * oc.tok_bytes) = (uint16_t)((i & 1) ? (yv >> 16) : (yv & 0xffffu));
+        if (oc.sa != nullptr) *reinterpret_cast<float*>(oc.sa + (size_t)oc.voff * 4 + 2 * i * oc.tok_bytes) = SA[i];
+      }
     }
   }
+  oc.y += CK * oc.tok_bytes;
+  if (oc.sa != nullptr) oc.sa += 2 * CK * oc.tok_bytes;
 }
 
 __device__ __forceinline__ void load_state(Consumer& C, const Wkv7Args& A, int64_t b, int64_t h) {
@@ -599,20 +615,43 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_fwd_kernel(Wk
   __syncthreads();
 
   if (wave < NCONS) {
+    // the chunk-to-chunk dependency runs through the consumers: let them issue ahead of the producers
+    __builtin_amdgcn_s_setprio(3);
     const bool q2drop = (A.flags & 1u) && L < A.T && A.ns != nullptr && A.ns[b * A.T + L] != 0;
     Consumer C;
     C.q = wave;
     C.lane = lane;
     load_state(C, A, b, h);
     if (L == 0) store_state0(C, A, b, h, q2drop);
-    for (int64_t c = 0; c < nchunks; ++c) {
-      const int64_t c0 = c * CK;
-      const int nvalid = (int)((A.T - c0 < CK) ? (A.T - c0) : CK);
-      const int si = (int)(c % RING);
-      wait_ready(sy, si, (int)c + 1);
-      consume(C, &slots[si], snapslot, A, b, h, c0, nvalid, q2drop);
-      // every LDS read of the slot has returned (its data was used above)
-      if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], (int)c + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    OutCursor oc;
+    oc.tok_bytes = (size_t)A.H * 64 * 2;
+    oc.y = reinterpret_cast<char*>(A.out) + (((size_t)b * A.T) * A.H + h) * 64 * 2;
+    oc.sa = A.sa ? reinterpret_cast<char*>(A.sa) + (((size_t)b * A.T) * A.H + h) * 64 * 4 : nullptr;
+    oc.voff = (uint32_t)((4 * (lane >> 4)) * (int)A.H * 64 + 16 * wave + (lane & 15));
+    const int csnap = L >= 1 ? (int)((L - 1) / CK) : -1;
+    const int nch = (int)nchunks;
+    // one chunk: consume with operand set `cur`, fetching the next chunk's set into `nxt` on the way
+    auto step = [&](int c, const Ops& cur, Ops& nxt) {
+      const int nvalid = (c + 1 < nch || A.T % CK == 0) ? CK : (int)(A.T % CK);
+      const int si = c % RING;
+      consume(C, cur, &slots[si], snapslot, A, b, h, nvalid, c == csnap, q2drop, oc, [&]() {
+        if (c + 1 < nch) {
+          const int sn = (c + 1) % RING;
+          wait_ready(sy, sn, c + 2);
+          load_ops(nxt, &slots[sn], wave, lane);
+        }
+      });
+      // every LDS read of slot si has returned: its data went into the MFMAs above
+      if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], c + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    };
+    Ops opA, opB;
+    if (nch > 0) {
+      wait_ready(sy, 0, 1);
+      load_ops(opA, &slots[0], wave, lane);
+    }
+    for (int c = 0; c < nch; c += 2) {
+      step(c, opA, opB);
+      if (c + 1 < nch) step(c + 1, opB, opA);
     }
   } else {
     const int p = wave - NCONS;
@@ -637,11 +676,8 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_fwd_kernel(Wk
       const int si = (int)(c % RING);
       Slot* slot = &slots[si];
       if (c >= RING) wait_consumed(sy, si, (int)(c - RING) + 1, lane);
-      prod_stage0(P, raw, F, slot, snapslot);
+      produce(P, raw, F, slot, snapslot);
       if (c + NPROD < nchunks) load_raw(raw, A, b, h, c0 + NPROD * CK, lane);
-      prod_stage1(P);
-      prod_stage2(P, F, slot);
-      prod_stage3(P, F, slot, snapslot);
       // the release orders this wave's LDS writes before the sequence number
       if (lane == 0) __hip_atomic_store(&sy->ready[si], (int)c + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
