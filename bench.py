@@ -1,10 +1,13 @@
-"""Benchmark of the WKV7 hot path on one MI355X:  python bench.py [--gpus 1] [--steps K] [--warmup W]
+"""Benchmark of the WKV hot path on one MI355X:  python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A step is one forward pass of the isolated WKV7 op over one synthetic batch of the headline shape
 (B=8, T=4096, H=32, N=64, bf16 I/O, fp32 state, new_starts ~ Bernoulli(1/1024), length ~ U{T/2..T}); inputs are
 resident in HBM before the timed region.  Prints ONE JSON line: forward tokens/s as `value`, forward+backward
 tokens/s beside it, the HBM roofline of the dominant kernel and a bounded CPU baseline (the oracle's
 associative-scan restatement on the host cores).
+
+`--workload wkv6` / `--workload wkv4` time the two secondary ops (B=16 T=2048 H=32 N=64 bf16, and B=32 T=4096
+C=2560 fp32) with the same JSON layout; the default, and the line the headline metric is quoted on, is wkv7.
 """
 import argparse
 import json
@@ -20,6 +23,9 @@ import numpy as np  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
 B, T, H, N = 8, 4096, 32, 64
+# HBM bytes per forward launch of the headline workload, from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`
+# (scaled by a 1 GiB copy; the summary with the commands is profiles/wkv7_fwd_bwd_B8_T4096_H32_bf16.md)
+WKV7_FWD_TRAFFIC_BYTES = 951.9e6
 
 
 def make_inputs(torch, seed=0):
@@ -43,20 +49,20 @@ def make_inputs(torch, seed=0):
 
 
 def time_region(torch, fn, steps, warmup):
-    """Wall time of exactly `steps` calls, bracketed by device syncs, plus per-call HIP-event durations."""
+    """Wall time of exactly `steps` calls, bracketed by device syncs, and the HIP-event time of the same region
+    (events recorded on the stream the kernels are launched on) divided by `steps`."""
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
-    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
-    for e0, e1 in evs:
-        e0.record()
+    e0.record()
+    for _ in range(steps):
         fn()
-        e1.record()
+    e1.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    per_call_ms = [e0.elapsed_time(e1) for e0, e1 in evs]
-    return wall, per_call_ms
+    return wall, e0.elapsed_time(e1) / steps
 
 
 def cpu_baseline(sample_heads=2, threads=None):
@@ -99,14 +105,120 @@ def cpu_baseline_sequential(tokens=1024):
             "sample": f"1 sequence, T={tokens}, all {H} heads, float64 sequential loop (oracle.wkv7.wkv7_base), {dt:.1f} s"}
 
 
+def base_record(metric, value, ms_step, args, dtype, workload, extra_config=None):
+    cfg = {"workload": workload}
+    cfg.update(extra_config or {})
+    return {"metric": metric, "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+            "warmup": args.warmup, "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak",
+            "vs_baseline": None, "dtype": dtype, "data": "synthetic", "config": cfg}
+
+
+def roofline(bytes_per_launch, kern_ms, traffic):
+    achieved = bytes_per_launch / (kern_ms * 1e-3) / 1e9
+    return {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
+            "traffic": traffic, "kernel_ms": kern_ms, "algorithmic_bytes": bytes_per_launch}
+
+
+def bench_wkv7(torch, ops, args):
+    x = make_inputs(torch)
+    tokens = B * T
+
+    def fwd():
+        return ops.wkv7_fwd(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], x["length"], x["new_starts"],
+                            compat=True, want_sa=False, force_seq=args.seq)
+
+    wall, kern_ms = time_region(torch, fwd, args.steps, args.warmup)
+    ms_step = 1e3 * wall / args.steps
+    # r,w,k,v,a,b in + y out (bf16), fp32 state in + out, new_starts, length
+    fwd_bytes = 7 * tokens * H * N * 2 + 2 * B * H * N * N * 4 + B * T + B * 4
+    out = base_record("WKV7 fwd tokens/s (B8 T4096 H32 N64 bf16)", tokens / (ms_step * 1e-3), ms_step, args, "bf16",
+                      "isolated WKV7 op, B=8 T=4096 H=32 N=64, bf16 r/w/k/v/a/b/y, fp32 state, "
+                      "new_starts~Bernoulli(1/1024), length~U{T/2..T} (BASELINE configs[1])",
+                      {"kernel": "sequential fp32 VALU" if args.seq else "chunked MFMA (bf16 hi+lo operands, fp32 accumulate)"})
+    out["roofline"] = roofline(fwd_bytes, kern_ms, None if args.seq else WKV7_FWD_TRAFFIC_BYTES)
+    if not args.no_bwd:
+        def fwd_bwd():
+            new_s, y, sa = ops.wkv7_fwd(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], x["length"],
+                                        x["new_starts"], compat=True, want_sa=True, force_seq=args.seq)
+            return ops.wkv7_bwd(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], x["length"], x["new_starts"],
+                                x["dy"], sa, None, compat=True)
+        n2 = max(2, args.steps // 4)
+        wall2, _ = time_region(torch, fwd_bwd, n2, 1)
+        ms2 = 1e3 * wall2 / n2
+        # forward (7 tensors) + backward reads r,w,k,v,a,b,dy and writes 6 gradients: 20 token tensors in bf16
+        fb_bytes = 20 * tokens * H * N * 2 + 4 * B * H * N * N * 4
+        out["fwd_bwd"] = {"tokens_per_s": tokens / (ms2 * 1e-3), "ms_per_step": ms2,
+                          "hbm_frac": fb_bytes / (ms2 * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": fb_bytes,
+                          "note": "backward = three sequential fp32 sweeps (no chunked MFMA backward yet)"}
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline()
+        out["cpu_baseline_sequential"] = cpu_baseline_sequential()
+        out["gpu_over_cpu"] = out["value"] / out["cpu_baseline"]["value"]
+    return out
+
+
+def bench_wkv6(torch, ops, args):
+    b6, t6 = 16, 2048
+    g = np.random.default_rng(0)
+    shp = (b6, t6, H, N)
+    f = lambda x: torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).cuda().bfloat16()
+    r, k, v, dy = (f(g.standard_normal(shp, dtype=np.float32)) for _ in range(4))
+    w = f(-np.exp(-0.5 + 0.5 * g.standard_normal(shp, dtype=np.float32)))
+    u = f(0.5 * g.standard_normal((H, N), dtype=np.float32))
+    s = torch.zeros((b6, H, N, N), dtype=torch.float32, device="cuda")
+    ns = torch.from_numpy(g.random((b6, t6)) < 1.0 / 512).cuda()
+    tokens = b6 * t6
+    fwd = lambda: ops.wkv6_fwd(r, k, v, w, u, s, None, ns, compat=True)
+    wall, kern_ms = time_region(torch, fwd, args.steps, args.warmup)
+    ms_step = 1e3 * wall / args.steps
+    fwd_bytes = 5 * tokens * H * N * 2 + 2 * b6 * H * N * N * 4 + b6 * t6
+    out = base_record("WKV6 fwd tokens/s (B16 T2048 H32 N64 bf16)", tokens / (ms_step * 1e-3), ms_step, args, "bf16",
+                      "isolated WKV6 op, B=16 T=2048 H=32 N=64 bf16, zero state, new_starts~Bernoulli(1/512) "
+                      "(BASELINE configs[2])", {"kernel": "sequential fp32 VALU"})
+    out["roofline"] = roofline(fwd_bytes, kern_ms, None)
+    if not args.no_bwd:
+        fb = lambda: ops.wkv6_bwd(r, k, v, w, u, s, None, ns, dy, None, compat=True)
+        n2 = max(2, args.steps // 4)
+        wall2, _ = time_region(torch, lambda: (fwd(), fb()), n2, 1)
+        ms2 = 1e3 * wall2 / n2
+        fb_bytes = 14 * tokens * H * N * 2 + 4 * b6 * H * N * N * 4
+        out["fwd_bwd"] = {"tokens_per_s": tokens / (ms2 * 1e-3), "ms_per_step": ms2,
+                          "hbm_frac": fb_bytes / (ms2 * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": fb_bytes}
+    return out
+
+
+def bench_wkv4(torch, ops, args):
+    b4, t4, c4 = 32, 4096, 2560
+    g = np.random.default_rng(0)
+    f = lambda x: torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).cuda()
+    k = f(g.standard_normal((b4, t4, c4), dtype=np.float32))
+    v = f(g.standard_normal((b4, t4, c4), dtype=np.float32))
+    w = f(-np.exp(g.standard_normal(c4, dtype=np.float32)))
+    u = f(0.5 * g.standard_normal(c4, dtype=np.float32))
+    s = torch.zeros((b4, 3, c4), dtype=torch.float32, device="cuda")
+    s[:, 2] = -1e38
+    length = torch.from_numpy(g.integers(1024, t4 + 1, size=(b4,)).astype(np.int32)).cuda()
+    tokens = b4 * t4
+    fwd = lambda: ops.wkv4_fwd(w, u, k, v, s, length, None, compat=True)
+    wall, kern_ms = time_region(torch, fwd, args.steps, args.warmup)
+    ms_step = 1e3 * wall / args.steps
+    fwd_bytes = 3 * tokens * c4 * 4 + 2 * b4 * 3 * c4 * 4
+    out = base_record("WKV4 fwd tokens/s (B32 T4096 C2560 fp32)", tokens / (ms_step * 1e-3), ms_step, args, "f32",
+                      "isolated WKV4 op, B=32 T=4096 C=2560 fp32, state (0,0,-1e38), length~U{1024..4096} "
+                      "(BASELINE configs[3])", {"kernel": "one thread per (sequence, channel)"})
+    out["roofline"] = roofline(fwd_bytes, kern_ms, None)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", choices=("wkv7", "wkv6", "wkv4"), default="wkv7")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-bwd", action="store_true")
-    ap.add_argument("--seq", action="store_true", help="force the sequential fp32 VALU kernel")
+    ap.add_argument("--seq", action="store_true", help="WKV7: force the sequential fp32 VALU kernel")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run three 1 GiB device copies before the timed region (scale for rocprofv3 --pmc)")
     args = ap.parse_args()
@@ -120,9 +232,6 @@ def main():
         print("bench.py needs a GPU", file=sys.stderr)
         sys.exit(2)
     _lib.load()
-    x = make_inputs(torch)
-    tokens = B * T
-
     if args.copy_probe:
         src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(1)
         dst = torch.empty_like(src)
@@ -130,45 +239,7 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-
-    def fwd():
-        return ops.wkv7_fwd(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], x["length"], x["new_starts"],
-                            compat=True, want_sa=False, force_seq=args.seq)
-
-    wall, per_call = time_region(torch, fwd, args.steps, args.warmup)
-    ms_step = 1e3 * wall / args.steps
-    kern_ms = float(np.mean(per_call))
-    fwd_bytes = 7 * tokens * H * N * 2 + 2 * B * H * N * N * 4 + B * T + B * 4
-    achieved = fwd_bytes / (kern_ms * 1e-3) / 1e9
-
-    out = {
-        "metric": "WKV7 fwd tokens/s (B8 T4096 H32 N64 bf16)", "value": tokens / (ms_step * 1e-3), "unit": "tokens/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_step,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16 I/O, fp32 state/accumulate",
-        "data": "synthetic",
-        "config": {"workload": "isolated WKV7 op, B=8 T=4096 H=32 N=64, bf16 r/w/k/v/a/b, fp32 state, "
-                               "new_starts~Bernoulli(1/1024), length~U{T/2..T} (BASELINE configs[1])",
-                   "kernel": "sequential" if args.seq else "default"},
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
-                     "kernel_ms": kern_ms, "algorithmic_bytes": fwd_bytes},
-    }
-
-    if not args.no_bwd:
-        def fwd_bwd():
-            new_s, y, sa = ops.wkv7_fwd(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], x["length"],
-                                        x["new_starts"], compat=True, want_sa=True)
-            return ops.wkv7_bwd(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], x["length"], x["new_starts"],
-                                x["dy"], sa, None, compat=True)
-        wall2, _ = time_region(torch, fwd_bwd, max(2, args.steps // 4), 1)
-        ms2 = 1e3 * wall2 / max(2, args.steps // 4)
-        fb_bytes = 20 * tokens * H * N * 2 + 4 * B * H * N * N * 4
-        out["fwd_bwd"] = {"tokens_per_s": tokens / (ms2 * 1e-3), "ms_per_step": ms2,
-                          "hbm_frac": fb_bytes / (ms2 * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": fb_bytes}
-    if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline()
-        out["cpu_baseline_sequential"] = cpu_baseline_sequential()
-        out["gpu_over_cpu"] = out["value"] / out["cpu_baseline"]["value"]
+    out = {"wkv7": bench_wkv7, "wkv6": bench_wkv6, "wkv4": bench_wkv4}[args.workload](torch, ops, args)
     print(json.dumps(out))
 
 
