@@ -523,7 +523,8 @@ __device__ __forceinline__ void consume(Consumer& C, const Ops& o, const Slot* _
     }
   }
   // state update, tile by tile: rows = keys.  S <- (S + Bh^T SA^T + Kh^T V^T) . gamma
-  if (!o.keep_end) {
+  if (__builtin_amdgcn_readfirstlane(o.keep_end) == 0) {
+    asm volatile("" ::: "memory");   // keep this a (rare, uniform) branch instead of 16 selects on the hot path
 #pragma unroll
     for (int tile = 0; tile < 4; ++tile) C.S[tile] = zero4;   // a reset inside the chunk cuts the entering state off
   }
