@@ -27,6 +27,9 @@ SIGNATURES = {
     "hiprwkv_wkv6_bwd": (_int, [_vp, _int, _int, _i64, _i64, _i64, _i64] + [_vp] * 6 + [_vp, _vp] + [_vp, _vp]
                          + [_vp] * 6 + [_vp, _sz, _u32]),
     "hiprwkv_wkv4_fwd": (_int, [_vp, _int, _i64, _i64, _i64] + [_vp] * 5 + [_vp, _vp] + [_vp, _vp, _u32]),
+    "hiprwkv_wkv4_bwd_workspace_bytes": (_sz, [_i64] * 3),
+    "hiprwkv_wkv4_bwd": (_int, [_vp, _int, _i64, _i64, _i64] + [_vp] * 6 + [_vp, _vp] + [_vp] + [_vp] * 5
+                         + [_vp, _sz, _u32]),
 }
 
 _lib = None

@@ -189,4 +189,36 @@ int hiprwkv_wkv4_fwd(hiprwkv_stream stream, int io_dtype, int64_t B, int64_t T, 
   return HIPRWKV_OK;
 }
 
+size_t hiprwkv_wkv4_bwd_workspace_bytes(int64_t B, int64_t T, int64_t C) {
+  return align256((size_t)B * ((T + 15) / 16) * 3 * C * sizeof(float));
+}
+
+int hiprwkv_wkv4_bwd(hiprwkv_stream stream, int io_dtype, int64_t B, int64_t T, int64_t C, const void* w,
+                     const void* u, const void* k, const void* v, const void* gy, const void* s,
+                     const uint32_t* length, const uint8_t* new_starts, const void* gs_new, float* gw, float* gu,
+                     void* gk, void* gv, void* gs, void* workspace, size_t workspace_bytes, unsigned flags) {
+  if (!dtype_ok(io_dtype)) return fail(HIPRWKV_EINVAL, "wkv4_bwd: dtype must be HIPRWKV_F32 or HIPRWKV_BF16");
+  if (B <= 0 || T <= 0 || C <= 0) return fail(HIPRWKV_EINVAL, "wkv4_bwd: B,T,C must be positive");
+  if (B * ((C + 63) / 64) > 0x7fffffffLL) return fail(HIPRWKV_EINVAL, "wkv4_bwd: B*C exceeds the grid limit");
+  const void* req[] = {w, u, k, v, gy, s, gw, gu, gk, gv, gs, workspace};
+  for (const void* p : req)
+    if (p == nullptr) return fail(HIPRWKV_EINVAL, "wkv4_bwd: null tensor pointer");
+  const size_t need = hiprwkv_wkv4_bwd_workspace_bytes(B, T, C);
+  if (workspace_bytes < need)
+    return fail(HIPRWKV_ENOSPACE, "wkv4_bwd: workspace has %zu bytes, %zu needed", workspace_bytes, need);
+  Wkv4Args A;
+  memset(&A, 0, sizeof(A));
+  A.B = B; A.T = T; A.C = C;
+  A.w = w; A.u = u; A.k = k; A.v = v; A.s = s;
+  A.length = length; A.ns = new_starts;
+  A.io_f32 = io_dtype == HIPRWKV_F32;
+  A.flags = flags;
+  A.gy = gy; A.gs_new = gs_new;
+  A.gk = gk; A.gv = gv; A.gs = gs; A.gw = gw; A.gu = gu;
+  A.ckpt = static_cast<float*>(workspace);
+  hipError_t e = launch_wkv4_bwd(A, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "wkv4_bwd: %s", hipGetErrorString(e));
+  return HIPRWKV_OK;
+}
+
 }  // extern "C"

@@ -100,6 +100,174 @@ __global__ __launch_bounds__(W4_THREADS) void wkv4_fwd_kernel(Wkv4Args A) {
   }
 }
 
+// ------------------------------------------------------------------ backward
+// Reverse-mode derivative of the recurrence above, step by step (so that it agrees with autodiff of the
+// reference's scan implementation, including how max() routes its cotangent).  The states entering each step are
+// needed in reverse order: a first kernel re-runs the recurrence and keeps the state entering every W4_SEG-th
+// step; the second kernel walks the segments backwards, recomputes the W4_SEG states of a segment into registers
+// and then differentiates its steps last to first.
+constexpr int W4_SEG = 16;
+
+template <typename IO>
+__global__ __launch_bounds__(W4_THREADS) void wkv4_ckpt_kernel(Wkv4Args A) {
+  const int64_t cblocks = (A.C + W4_THREADS - 1) / W4_THREADS;
+  const int64_t b = blockIdx.x / cblocks;
+  const int64_t c = (blockIdx.x % cblocks) * W4_THREADS + threadIdx.x;
+  if (c >= A.C) return;
+  const IO* kp = reinterpret_cast<const IO*>(A.k) + (size_t)b * A.T * A.C + c;
+  const IO* vp = reinterpret_cast<const IO*>(A.v) + (size_t)b * A.T * A.C + c;
+  const IO* sp = reinterpret_cast<const IO*>(A.s) + (size_t)b * 3 * A.C + c;
+  const uint8_t* ns = A.ns ? A.ns + (size_t)b * A.T : nullptr;
+  const int64_t nseg = (A.T + W4_SEG - 1) / W4_SEG;
+  float* ck = A.ckpt + (size_t)b * nseg * 3 * A.C + c;
+  const float w = ld_f(reinterpret_cast<const IO*>(A.w) + c);
+  float aa = ld_f(sp), bb = ld_f(sp + A.C), pp = ld_f(sp + 2 * A.C);
+  for (int64_t sg = 0; sg < nseg; ++sg) {
+    ck[(sg * 3 + 0) * A.C] = aa;
+    ck[(sg * 3 + 1) * A.C] = bb;
+    ck[(sg * 3 + 2) * A.C] = pp;
+    float kc[W4_SEG], vc[W4_SEG];
+#pragma unroll
+    for (int x = 0; x < W4_SEG; ++x) {
+      const int64_t t = sg * W4_SEG + x;
+      kc[x] = t < A.T ? ld_f(kp + (size_t)t * A.C) : 0.f;
+      vc[x] = t < A.T ? ld_f(vp + (size_t)t * A.C) : 0.f;
+    }
+#pragma unroll
+    for (int x = 0; x < W4_SEG; ++x) {
+      const int64_t t = sg * W4_SEG + x;
+      if (t < A.T) {
+        if (ns != nullptr && ns[t]) { aa = 0.f; bb = 0.f; pp = W4_RESET_PP; }
+        const float ww = pp + w, diff = ww - kc[x];
+        const float e = __expf(-fabsf(diff));
+        const float e1 = diff >= 0.f ? 1.f : e, e2 = diff >= 0.f ? e : 1.f;
+        aa = fmaf(e1, aa, e2 * vc[x]);
+        bb = fmaf(e1, bb, e2);
+        pp = fmaxf(ww, kc[x]);
+      }
+    }
+  }
+}
+
+template <typename IO>
+__global__ __launch_bounds__(W4_THREADS) void wkv4_bwd_kernel(Wkv4Args A) {
+  const int64_t cblocks = (A.C + W4_THREADS - 1) / W4_THREADS;
+  const int64_t b = blockIdx.x / cblocks;
+  const int64_t c = (blockIdx.x % cblocks) * W4_THREADS + threadIdx.x;
+  if (c >= A.C) return;
+  const size_t tok0 = (size_t)b * A.T * A.C + c;
+  const IO* kp = reinterpret_cast<const IO*>(A.k) + tok0;
+  const IO* vp = reinterpret_cast<const IO*>(A.v) + tok0;
+  const IO* gyp = reinterpret_cast<const IO*>(A.gy) + tok0;
+  IO* gkp = reinterpret_cast<IO*>(A.gk) + tok0;
+  IO* gvp = reinterpret_cast<IO*>(A.gv) + tok0;
+  const uint8_t* ns = A.ns ? A.ns + (size_t)b * A.T : nullptr;
+  const int64_t nseg = (A.T + W4_SEG - 1) / W4_SEG;
+  const float* ck = A.ckpt + (size_t)b * nseg * 3 * A.C + c;
+  const float w = ld_f(reinterpret_cast<const IO*>(A.w) + c);
+  const float u = ld_f(reinterpret_cast<const IO*>(A.u) + c);
+  int64_t L = A.length ? (int64_t)A.length[b] : A.T;
+  L = L < A.T ? L : A.T;
+  const bool q2drop = (A.flags & 1u) && L < A.T && ns != nullptr && ns[L] != 0;
+  float inj_a = 0.f, inj_b = 0.f, inj_p = 0.f;   // cotangent of the returned state
+  if (A.gs_new != nullptr && !q2drop) {
+    const IO* gp = reinterpret_cast<const IO*>(A.gs_new) + (size_t)b * 3 * A.C + c;
+    inj_a = ld_f(gp); inj_b = ld_f(gp + A.C); inj_p = ld_f(gp + 2 * A.C);
+  }
+  float g_aa = 0.f, g_bb = 0.f, g_pp = 0.f, gw = 0.f, gu = 0.f;
+  for (int64_t sg = nseg - 1; sg >= 0; --sg) {
+    const int64_t t0 = sg * W4_SEG;
+    float kc[W4_SEG], vc[W4_SEG], gc[W4_SEG], sa[W4_SEG], sb[W4_SEG], spp[W4_SEG];
+    uint32_t rmask = 0;
+#pragma unroll
+    for (int x = 0; x < W4_SEG; ++x) {
+      const int64_t t = t0 + x;
+      const bool in = t < A.T;
+      kc[x] = in ? ld_f(kp + (size_t)t * A.C) : 0.f;
+      vc[x] = in ? ld_f(vp + (size_t)t * A.C) : 0.f;
+      gc[x] = in ? ld_f(gyp + (size_t)t * A.C) : 0.f;
+      if (in && ns != nullptr && ns[t]) rmask |= 1u << x;
+    }
+    float aa = ck[(sg * 3 + 0) * A.C], bb = ck[(sg * 3 + 1) * A.C], pp = ck[(sg * 3 + 2) * A.C];
+    // states entering each step of the segment
+#pragma unroll
+    for (int x = 0; x < W4_SEG; ++x) {
+      if (rmask & (1u << x)) { aa = 0.f; bb = 0.f; pp = W4_RESET_PP; }
+      sa[x] = aa; sb[x] = bb; spp[x] = pp;
+      const float ww = pp + w, diff = ww - kc[x];
+      const float e = __expf(-fabsf(diff));
+      const float e1 = diff >= 0.f ? 1.f : e, e2 = diff >= 0.f ? e : 1.f;
+      aa = fmaf(e1, aa, e2 * vc[x]);
+      bb = fmaf(e1, bb, e2);
+      pp = fmaxf(ww, kc[x]);
+    }
+#pragma unroll
+    for (int x = W4_SEG - 1; x >= 0; --x) {
+      const int64_t t = t0 + x;
+      if (t < A.T) {
+        if (t == L - 1) { g_aa += inj_a; g_bb += inj_b; g_pp += inj_p; }
+        const float a0 = sa[x], b0 = sb[x], p0 = spp[x], kt = kc[x], vt = vc[x], gy = gc[x];
+        // state update: aa' = f1 aa + f2 v, bb' = f1 bb + f2, pp' = max(pp + w, k)
+        const float ww2 = p0 + w, d2 = ww2 - kt;
+        const float ex2 = __expf(-fabsf(d2));
+        const bool up2 = d2 >= 0.f;
+        const float f1 = up2 ? 1.f : ex2, f2 = up2 ? ex2 : 1.f;
+        const float gf1 = (g_aa * a0 + g_bb * b0) * f1, gf2 = (g_aa * vt + g_bb) * f2;
+        float n_aa = g_aa * f1, n_bb = g_bb * f1;
+        float gv = g_aa * f2;
+        const float gq2 = g_pp - gf1 - gf2;
+        const float gww2 = gf1 + (up2 ? gq2 : 0.f);
+        float gk = gf2 + (up2 ? 0.f : gq2);
+        float n_pp = gww2;
+        gw += gww2;
+        // output: y = (e1 aa + e2 v) / (e1 bb + e2) with q = max(pp, u + k)
+        const float ww = u + kt, d1 = p0 - ww;
+        const float ex1 = __expf(-fabsf(d1));
+        const bool up1 = d1 >= 0.f;
+        const float e1 = up1 ? 1.f : ex1, e2 = up1 ? ex1 : 1.f;
+        const float An = fmaf(e1, a0, e2 * vt), Bd = fmaf(e1, b0, e2);
+        const float rB = __frcp_rn(Bd);
+        const float gA = gy * rB, gB = -gy * An * rB * rB;
+        const float ge1 = (gA * a0 + gB * b0) * e1, ge2 = (gA * vt + gB) * e2;
+        n_aa = fmaf(gA, e1, n_aa);
+        n_bb = fmaf(gB, e1, n_bb);
+        gv = fmaf(gA, e2, gv);
+        const float gq = -ge1 - ge2;
+        n_pp += ge1 + (up1 ? gq : 0.f);
+        const float gww = ge2 + (up1 ? 0.f : gq);
+        gu += gww;
+        gk += gww;
+        st_f(gkp + (size_t)t * A.C, gk);
+        st_f(gvp + (size_t)t * A.C, gv);
+        const bool reset = (rmask >> x) & 1u;
+        g_aa = reset ? 0.f : n_aa;
+        g_bb = reset ? 0.f : n_bb;
+        g_pp = reset ? 0.f : n_pp;
+      }
+    }
+  }
+  if (L == 0) { g_aa += inj_a; g_bb += inj_b; g_pp += inj_p; }   // the returned state is the input state itself
+  IO* gsp = reinterpret_cast<IO*>(A.gs) + (size_t)b * 3 * A.C + c;
+  st_f(gsp, g_aa);
+  st_f(gsp + A.C, g_bb);
+  st_f(gsp + 2 * A.C, g_pp);
+  A.gw[(size_t)b * A.C + c] = gw;
+  A.gu[(size_t)b * A.C + c] = gu;
+}
+
+hipError_t launch_wkv4_bwd(const Wkv4Args& A, hipStream_t stream) {
+  const int64_t cblocks = (A.C + W4_THREADS - 1) / W4_THREADS;
+  const dim3 grid((unsigned)(A.B * cblocks)), block(W4_THREADS);
+  if (A.io_f32) {
+    hipLaunchKernelGGL(wkv4_ckpt_kernel<float>, grid, block, 0, stream, A);
+    hipLaunchKernelGGL(wkv4_bwd_kernel<float>, grid, block, 0, stream, A);
+  } else {
+    hipLaunchKernelGGL(wkv4_ckpt_kernel<bf16_t>, grid, block, 0, stream, A);
+    hipLaunchKernelGGL(wkv4_bwd_kernel<bf16_t>, grid, block, 0, stream, A);
+  }
+  return hipGetLastError();
+}
+
 hipError_t launch_wkv4_fwd(const Wkv4Args& A, hipStream_t stream) {
   const int64_t cblocks = (A.C + W4_THREADS - 1) / W4_THREADS;
   const dim3 grid((unsigned)(A.B * cblocks)), block(W4_THREADS);

@@ -50,6 +50,12 @@ struct Wkv4Args {
   void* out;
   int io_f32;
   unsigned flags;
+  // backward only
+  const void* gy;
+  const void* gs_new;
+  void *gk, *gv, *gs;
+  float *gw, *gu;   // (B,C) each
+  float* ckpt;      // workspace: (B, ceil(T/16), 3, C) states entering every 16th step
 };
 
 hipError_t launch_wkv7_seq_fwd(const Wkv7Args& A, hipStream_t stream);
@@ -58,5 +64,6 @@ hipError_t launch_wkv7_seq_bwd(const Wkv7Args& A, hipStream_t stream);
 hipError_t launch_wkv6_seq_fwd(const Wkv6Args& A, hipStream_t stream);
 hipError_t launch_wkv6_seq_bwd(const Wkv6Args& A, hipStream_t stream);
 hipError_t launch_wkv4_fwd(const Wkv4Args& A, hipStream_t stream);
+hipError_t launch_wkv4_bwd(const Wkv4Args& A, hipStream_t stream);
 
 }  // namespace hiprwkv

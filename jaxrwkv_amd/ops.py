@@ -201,3 +201,50 @@ def wkv4_fwd(w_neg, u, k, v, s, length=None, new_starts=None, compat=True):
                               _p(new_starts), _p(new_s), _p(y), _flags(compat))
     _lib.check(rc, "hiprwkv_wkv4_fwd")
     return new_s, y
+
+
+def wkv4_bwd(w_neg, u, k, v, s, length, new_starts, gy, gs_new=None, compat=True):
+    """Cotangents (gw, gu, gk, gv, gs) of ``wkv4_fwd``; gw, gu are summed over the batch here (rwkv4.py:351)."""
+    lib = _lib.load()
+    io = k.dtype
+    k, v, s, w_neg, u, gy = (_dev(x, io) for x in (k, v, s, w_neg, u, gy))
+    gs_new = None if gs_new is None else _dev(gs_new, io)
+    B, T, C = k.shape
+    length, new_starts = _length_ns(length, new_starts, B, T, k.device)
+    gk, gv = torch.empty_like(k), torch.empty_like(v)
+    gs = torch.empty_like(s)
+    gw = torch.empty((B, C), dtype=torch.float32, device=k.device)
+    gu = torch.empty((B, C), dtype=torch.float32, device=k.device)
+    nbytes = lib.hiprwkv_wkv4_bwd_workspace_bytes(B, T, C)
+    ws = torch.empty(nbytes, dtype=torch.uint8, device=k.device)
+    rc = lib.hiprwkv_wkv4_bwd(_stream(), _DT[io], B, T, C, _p(w_neg), _p(u), _p(k), _p(v), _p(gy), _p(s), _p(length),
+                              _p(new_starts), _p(gs_new), _p(gw), _p(gu), _p(gk), _p(gv), _p(gs), _p(ws), nbytes,
+                              _flags(compat))
+    _lib.check(rc, "hiprwkv_wkv4_bwd")
+    return gw.sum(0).to(io), gu.sum(0).to(io), gk, gv, gs
+
+
+class _Wkv4(torch.autograd.Function):
+    """custom VJP, the counterpart of ``wkv4_cuda`` (rwkv4.py:379-383)."""
+
+    @staticmethod
+    def forward(ctx, w_neg, u, k, v, s, length, new_starts, compat):
+        new_s, y = wkv4_fwd(w_neg, u, k, v, s, length, new_starts, compat)
+        ctx.compat = compat
+        ctx.save_for_backward(w_neg, u, k, v, s, length, new_starts)
+        return new_s, y
+
+    @staticmethod
+    def backward(ctx, gs_new, gy):
+        w_neg, u, k, v, s, length, new_starts = ctx.saved_tensors
+        if gy is None:
+            gy = torch.zeros_like(k)
+        gw, gu, gk, gv, gs = wkv4_bwd(w_neg, u, k, v, s, length, new_starts, gy, gs_new, ctx.compat)
+        return gw, gu, gk, gv, gs, None, None, None
+
+
+def wkv4(w_neg, u, k, v, s, length=None, new_starts=None, compat=True):
+    """Differentiable WKV4 in the op's convention (w_neg = -exp(time_decay), no receptance): returns (new_s, wkv)."""
+    B, T = k.shape[:2]
+    length, new_starts = _length_ns(length, new_starts, B, T, k.device)
+    return _Wkv4.apply(w_neg, u, k, v, s, length, new_starts, compat)

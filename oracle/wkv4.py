@@ -115,3 +115,83 @@ def wkv4_assoc_literal(r, k, v, time_decay, time_first, s, length=None, new_star
         L = int(length[bi])
         out_s[bi] = np.stack([sA[L], sB[L], sP[L]])                        # :300
     return out_s, out
+
+
+def wkv4_ffi_bwd(w_neg, u, k, v, s, length, new_starts, gy, gs_new, compat=False):
+    """Reverse-mode derivative of ``wkv4_ffi`` step by step through the max-tracked recurrence (the program of
+    rwkv4.py:147-171, so that it agrees with autodiff of the reference's ScanRWKV): cotangents gy of the
+    un-gated output and gs_new of the returned raw state (aa, bb, pp).
+
+    Returns (gw (B,C), gu (B,C), gk, gv, gs (B,3,C)); gw and gu are per sequence, to be summed over B by the
+    caller as the reference does (rwkv4.py:351).  ``max`` passes its cotangent to the larger argument.
+    """
+    k, v, s, length, new_starts = _prep(k, v, s, length, new_starts)
+    w = np.asarray(w_neg, np.float64)
+    u = np.asarray(u, np.float64)
+    gy = np.asarray(gy, np.float64)
+    gs_new = np.asarray(gs_new, np.float64).copy()
+    B, T, C = k.shape
+    gs_extra = np.zeros_like(s)
+    for bi in range(B):
+        L = int(length[bi])
+        if compat and L < T and new_starts[bi, L]:
+            gs_new[bi] = 0.0
+        if L == 0:
+            gs_extra[bi] = gs_new[bi]
+            gs_new[bi] = 0.0
+    # forward sweep keeping the state entering every step
+    st = np.zeros((T, B, 3, C))
+    aa, bb, pp = s[:, 0].copy(), s[:, 1].copy(), s[:, 2].copy()
+    for t in range(T):
+        ns = new_starts[:, t, None]
+        aa, bb, pp = np.where(ns, 0.0, aa), np.where(ns, 0.0, bb), np.where(ns, RESET_PP, pp)
+        st[t, :, 0], st[t, :, 1], st[t, :, 2] = aa, bb, pp
+        ww = pp + w
+        qq = np.maximum(ww, k[:, t])
+        f1, f2 = np.exp(ww - qq), np.exp(k[:, t] - qq)
+        aa, bb, pp = f1 * aa + f2 * v[:, t], f1 * bb + f2, qq
+    gk, gv = np.zeros_like(k), np.zeros_like(v)
+    gw, gu = np.zeros((B, C)), np.zeros((B, C))
+    g_aa, g_bb, g_pp = np.zeros((B, C)), np.zeros((B, C)), np.zeros((B, C))
+    for t in range(T - 1, -1, -1):
+        inj = (length - 1 == t)[:, None]
+        g_aa = g_aa + np.where(inj, gs_new[:, 0], 0.0)
+        g_bb = g_bb + np.where(inj, gs_new[:, 1], 0.0)
+        g_pp = g_pp + np.where(inj, gs_new[:, 2], 0.0)
+        aa, bb, pp = st[t, :, 0], st[t, :, 1], st[t, :, 2]
+        kt, vt = k[:, t], v[:, t]
+        # state update
+        ww2 = pp + w
+        q2 = np.maximum(ww2, kt)
+        f1, f2 = np.exp(ww2 - q2), np.exp(kt - q2)
+        g_f1 = g_aa * aa + g_bb * bb
+        g_f2 = g_aa * vt + g_bb
+        n_aa, n_bb = g_aa * f1, g_bb * f1
+        g_v = g_aa * f2
+        g_q2 = g_pp - g_f1 * f1 - g_f2 * f2
+        g_ww2 = g_f1 * f1 + np.where(ww2 >= kt, g_q2, 0.0)
+        g_k = g_f2 * f2 + np.where(ww2 >= kt, 0.0, g_q2)
+        n_pp = g_ww2
+        gw += g_ww2
+        # output
+        ww = u + kt
+        q = np.maximum(pp, ww)
+        e1, e2 = np.exp(pp - q), np.exp(ww - q)
+        A, Bd = e1 * aa + e2 * vt, e1 * bb + e2
+        g_A = gy[:, t] / Bd
+        g_B = -gy[:, t] * A / (Bd * Bd)
+        g_e1 = g_A * aa + g_B * bb
+        g_e2 = g_A * vt + g_B
+        n_aa += g_A * e1
+        n_bb += g_B * e1
+        g_v += g_A * e2
+        g_q = -g_e1 * e1 - g_e2 * e2
+        n_pp += g_e1 * e1 + np.where(pp >= ww, g_q, 0.0)
+        g_ww = g_e2 * e2 + np.where(pp >= ww, 0.0, g_q)
+        gu += g_ww
+        g_k += g_ww
+        gk[:, t], gv[:, t] = g_k, g_v
+        ns = new_starts[:, t, None]
+        g_aa, g_bb, g_pp = np.where(ns, 0.0, n_aa), np.where(ns, 0.0, n_bb), np.where(ns, 0.0, n_pp)
+    gs = np.stack([g_aa, g_bb, g_pp], axis=1) + gs_extra
+    return gw, gu, gk, gv, gs

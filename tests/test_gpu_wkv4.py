@@ -73,3 +73,45 @@ def test_plugin_class_applies_decay_and_receptance():
     ref_s, ref_y = o4.wkv4_assoc_literal(r[None], x["k"], x["v"], td, x["u"], x["s"], x["length"], x["new_starts"])
     assert_close("out", host(out), ref_y[0])
     state_close(host(new_s)[None], ref_s)
+
+
+def run_bwd(x, gy, gs, compat):
+    from jaxrwkv_amd import ops
+    t = {n: dev(x[n]).requires_grad_() for n in ("w", "u", "k", "v", "s")}
+    new_s, y = ops.wkv4(t["w"], t["u"], t["k"], t["v"], t["s"], dev(x["length"]), dev(x["new_starts"]), compat=compat)
+    # the constant "minus infinity" of a reset state is excluded from the loss, as in the oracle's check
+    mask = (new_s > -1e29).float()
+    ((y * dev(gy)).sum() + (new_s * mask * dev(gs)).sum()).backward()
+    torch.cuda.synchronize()
+    return [host(t[n].grad) for n in ("w", "u", "k", "v", "s")]
+
+
+@pytest.mark.parametrize("compat", [True, False])
+@pytest.mark.parametrize("B,T,C,seed", [(2, 40, 64, 31), (3, 130, 100, 32), (1, 1, 64, 33)])
+def test_fp32_backward(B, T, C, seed, compat):
+    x = wkv4_inputs(B, T, C, seed=seed, p_reset=0.04, default_state=False, min_len=1)
+    if T > 4:
+        x["length"][0] = T // 2
+        x["new_starts"][0, T // 2] = True
+    g = np.random.default_rng(seed)
+    gy, gs = g.standard_normal(x["k"].shape), g.standard_normal(x["s"].shape)
+    ref_s, _ = o4.wkv4_ffi(x["w"], x["u"], x["k"], x["v"], x["s"], x["length"], x["new_starts"], compat=compat)
+    gs_eff = np.where(ref_s > -1e29, gs, 0.0)
+    gw, gu, gk, gv, gsi = o4.wkv4_ffi_bwd(x["w"], x["u"], x["k"], x["v"], x["s"], x["length"], x["new_starts"], gy, gs_eff, compat=compat)
+    got = run_bwd(x, gy, gs, compat)
+    for name, g_, rf in zip(("w", "u", "k", "v", "s"), got, (gw.sum(0), gu.sum(0), gk, gv, gsi)):
+        assert_close("g" + name, g_, rf, rtol=1e-4, atol=2e-5, scale_atol=True)
+
+
+def test_backward_length_zero_and_default_state():
+    x = wkv4_inputs(2, 20, 64, seed=34, p_reset=0.1)
+    x["length"][:] = 0
+    g = np.random.default_rng(1)
+    gy, gs = g.standard_normal(x["k"].shape), g.standard_normal(x["s"].shape)
+    for compat in (True, False):
+        ref_s, _ = o4.wkv4_ffi(x["w"], x["u"], x["k"], x["v"], x["s"], x["length"], x["new_starts"], compat=compat)
+        gs_eff = np.where(ref_s > -1e29, gs, 0.0)
+        gw, gu, gk, gv, gsi = o4.wkv4_ffi_bwd(x["w"], x["u"], x["k"], x["v"], x["s"], x["length"], x["new_starts"], gy, gs_eff, compat=compat)
+        got = run_bwd(x, gy, gs, compat)
+        for name, g_, rf in zip(("w", "u", "k", "v", "s"), got, (gw.sum(0), gu.sum(0), gk, gv, gsi)):
+            assert_close("g" + name, g_, rf, rtol=1e-4, atol=2e-5, scale_atol=True)

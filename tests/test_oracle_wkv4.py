@@ -81,3 +81,64 @@ def test_large_k_is_stable():
     _, y = o4.wkv4_ffi(x["w"], x["u"], k, x["v"], x["s"])
     assert np.all(np.isfinite(y))
     assert np.all(np.abs(y) <= np.abs(x["v"]).max() + 1e-9)      # a convex combination of the v's
+
+
+def _loss4(x, gy, gs, compat, **over):
+    q = dict(x)
+    q.update(over)
+    out_s, y = o4.wkv4_ffi(q["w"], q["u"], q["k"], q["v"], q["s"], q["length"], q["new_starts"], compat=compat)
+    out_s = np.where(out_s <= -1e29, 0.0, out_s)      # the constant "minus infinity" of a reset state would swamp the sum
+    return np.sum(y * gy) + np.sum(out_s * gs)
+
+
+@pytest.mark.parametrize("compat", [False, True])
+@pytest.mark.parametrize("case", ["plain", "len_at_reset", "len0"])
+def test_bwd_matches_finite_differences(compat, case):
+    x = wkv4_inputs(2, 9, 5, seed=11, p_reset=0.25, default_state=False, min_len=2)
+    x["new_starts"][0, 4] = True
+    if case == "len_at_reset":
+        x["length"][0] = 4
+    if case == "len0":
+        x["length"][:] = 0
+    g = np.random.default_rng(5)
+    gy, gs = g.standard_normal(x["k"].shape), g.standard_normal(x["s"].shape)
+    gw, gu, gk, gv, gsi = o4.wkv4_ffi_bwd(x["w"], x["u"], x["k"], x["v"], x["s"], x["length"], x["new_starts"], gy, gs, compat=compat)
+    grads = dict(w=gw.sum(0), u=gu.sum(0), k=gk, v=gv, s=gsi)
+    eps = 1e-6
+    for name, an in grads.items():
+        for _ in range(12):
+            idx = tuple(g.integers(0, n) for n in x[name].shape)
+            xp, xm = x[name].copy(), x[name].copy()
+            xp[idx] += eps
+            xm[idx] -= eps
+            fd = (_loss4(x, gy, gs, compat, **{name: xp}) - _loss4(x, gy, gs, compat, **{name: xm})) / (2 * eps)
+            assert abs(fd - an[idx]) < 2e-6 * max(1.0, abs(fd)), (name, idx, fd, an[idx])
+
+
+def test_bwd_matches_torch_autograd():
+    import torch
+    x = wkv4_inputs(2, 11, 6, seed=12, p_reset=0.2, default_state=False, min_len=3)
+    g = np.random.default_rng(6)
+    gy, gs = g.standard_normal(x["k"].shape), g.standard_normal(x["s"].shape)
+    tt = {n: torch.tensor(x[n], dtype=torch.float64, requires_grad=True) for n in ("w", "u", "k", "v", "s")}
+    ns, L = torch.tensor(x["new_starts"]), torch.tensor(x["length"])
+    aa, bb, pp = tt["s"][:, 0], tt["s"][:, 1], tt["s"][:, 2]
+    out_s, ys = tt["s"], []
+    for t in range(11):
+        keep = (~ns[:, t]).double()[:, None]
+        aa, bb, pp = aa * keep, bb * keep, pp * keep + (1 - keep) * o4.RESET_PP
+        kt, vt = tt["k"][:, t], tt["v"][:, t]
+        # written with logaddexp-style primitives rather than the oracle's explicit e1/e2
+        ww = tt["u"] + kt
+        q = torch.maximum(pp, ww)
+        ys.append((torch.exp(pp - q) * aa + torch.exp(ww - q) * vt) / (torch.exp(pp - q) * bb + torch.exp(ww - q)))
+        ww2 = pp + tt["w"]
+        q2 = torch.maximum(ww2, kt)
+        aa, bb, pp = torch.exp(ww2 - q2) * aa + torch.exp(kt - q2) * vt, torch.exp(ww2 - q2) * bb + torch.exp(kt - q2), q2
+        snap = (t < L).double()[:, None, None]
+        out_s = snap * torch.stack([aa, bb, pp], 1) + (1 - snap) * out_s
+    y = torch.stack(ys, 1)
+    ((y * torch.tensor(gy)).sum() + (out_s * torch.tensor(gs)).sum()).backward()
+    gw, gu, gk, gv, gsi = o4.wkv4_ffi_bwd(x["w"], x["u"], x["k"], x["v"], x["s"], x["length"], x["new_starts"], gy, gs)
+    for name, an in (("w", gw.sum(0)), ("u", gu.sum(0)), ("k", gk), ("v", gv), ("s", gsi)):
+        np.testing.assert_allclose(tt[name].grad.numpy(), an, rtol=1e-9, atol=1e-10, err_msg=name)
