@@ -412,8 +412,9 @@ struct Consumer {
   int q, lane;
 };
 
-// Operands a consumer needs at the start of a chunk; they are fetched from the slot while the previous chunk
-// is still being finished, so that their LDS latency is off the chunk-to-chunk dependency chain.
+// Operands a consumer carries from one chunk to the next.  Each group is reloaded for the next chunk right
+// after its last use in the current one, so the LDS latency hides behind the rest of the chunk and no second set
+// of registers is needed.
 struct Ops {
   u32x4_t aq[2][2][2];     // [hi|lo][At|Qt][j]: rows in the key order of the state tiles
   u32x4_t T, Ka, Br, Kr;   // T, Mka, Mbr, Mkr: hi pair, lo pair
@@ -421,7 +422,7 @@ struct Ops {
   int keep_end;
 };
 
-__device__ __forceinline__ void load_ops(Ops& o, const Slot* __restrict__ slot, int q, int lane) {
+__device__ __forceinline__ void load_aq(Ops& o, const Slot* __restrict__ slot, int q, int lane) {
   const int n = lane & 15, g = lane >> 4;
 #pragma unroll
   for (int pl = 0; pl < 2; ++pl)
@@ -430,13 +431,16 @@ __device__ __forceinline__ void load_ops(Ops& o, const Slot* __restrict__ slot, 
 #pragma unroll
       for (int j = 0; j < 2; ++j)
         o.aq[pl][ar][j] = *reinterpret_cast<const u32x4_t*>(&slot->AQ[pl][ar][n][32 * j + 8 * g]);
-  o.T = *reinterpret_cast<const u32x4_t*>(&slot->Mt[0][lane]);
   o.Ka = *reinterpret_cast<const u32x4_t*>(&slot->Mt[1][lane]);
-  o.Br = *reinterpret_cast<const u32x4_t*>(&slot->Mt[2][lane]);
   o.Kr = *reinterpret_cast<const u32x4_t*>(&slot->Mt[3][lane]);
-  const uint2 v0 = slot->VT[q][lane], v1 = slot->VT[q][lane];
-  o.vv = u32x4_t{v0.x, v0.y, v1.x, v1.y};
+  const uint2 v0 = slot->VT[q][lane];
+  o.vv = u32x4_t{v0.x, v0.y, v0.x, v0.y};
   o.keep_end = slot->keep_end;
+}
+__device__ __forceinline__ void load_ops(Ops& o, const Slot* __restrict__ slot, int q, int lane) {
+  load_aq(o, slot, q, lane);
+  o.T = *reinterpret_cast<const u32x4_t*>(&slot->Mt[0][lane]);
+  o.Br = *reinterpret_cast<const u32x4_t*>(&slot->Mt[2][lane]);
 }
 
 // Uniform output cursors of a consumer, advanced by one chunk per call.
@@ -447,12 +451,13 @@ struct OutCursor {
   uint32_t voff;       // lane part of the address, in elements: (4g * H) * 64 + value
 };
 
-// The S0-dependent part of one chunk.  `prefetch` runs once the update MFMAs are in flight: the caller uses it
-// to wait for, and fetch, the next chunk's operands.
-template <class Prefetch>
-__device__ __forceinline__ void consume(Consumer& C, const Ops& o, const Slot* __restrict__ slot,
-                                        const SnapSlot* __restrict__ snapslot, const Wkv7Args& A, int64_t b, int64_t h,
-                                        int nvalid, bool is_snap, bool q2drop, OutCursor& oc, Prefetch&& prefetch) {
+// The S0-dependent part of one chunk.  `next` is the slot of the following chunk (null after the last one);
+// `next_ready` waits until its producer has published it.
+template <class WaitNext>
+__device__ __forceinline__ void consume(Consumer& C, Ops& o, const Slot* __restrict__ slot,
+                                        const Slot* __restrict__ next, const SnapSlot* __restrict__ snapslot,
+                                        const Wkv7Args& A, int64_t b, int64_t h, int nvalid, bool is_snap, bool q2drop,
+                                        OutCursor& oc, WaitNext&& next_ready) {
   const int lane = C.lane, n = lane & 15, g = lane >> 4;
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
   // update operands of this chunk: needed last, so their latency hides behind the W / SA chain
@@ -464,6 +469,7 @@ __device__ __forceinline__ void consume(Consumer& C, const Ops& o, const Slot* _
     bt[1][tile] = *reinterpret_cast<const u32x4_t*>(&slot->BT[1][tile][lane]);
     gm[tile] = *reinterpret_cast<const float4*>(&slot->gamma[16 * tile + 4 * g]);
   }
+  const bool keep_end = __builtin_amdgcn_readfirstlane(o.keep_end) != 0;
   // B operands from the state: MFMA j contracts over the keys of tiles 2j and 2j+1
   u32x4_t Sh[2], Sl[2];
 #pragma unroll
@@ -483,6 +489,12 @@ __device__ __forceinline__ void consume(Consumer& C, const Ops& o, const Slot* _
   }
   W = mfma(o.Ka, o.vv, W);                    // W += Mka^T V^T (hi and lo parts side by side)
   Y = mfma(o.Kr, o.vv, Y);                    // Y += Mkr^T V^T
+  const u32x4_t vv = o.vv;
+  // At, Qt, Mka, Mkr, v^T are dead now: fetch the next chunk's into the same registers
+  if (next != nullptr) {
+    next_ready();
+    load_aq(o, next, C.q, lane);
+  }
   uint32_t h0, l0, h1, l1;
   split2(W[0], W[1], h0, l0);
   split2(W[2], W[3], h1, l1);
@@ -494,11 +506,13 @@ __device__ __forceinline__ void consume(Consumer& C, const Ops& o, const Slot* _
     SA = mfma(o.T, bhh, zero4);               // (T_hi + T_lo)^T W_hi
     SA = mfma(o.T, bl0, SA);                  // T_hi^T W_lo
   }
+  if (next != nullptr) o.T = *reinterpret_cast<const u32x4_t*>(&next->Mt[0][lane]);
   split2(SA[0], SA[1], h0, l0);
   split2(SA[2], SA[3], h1, l1);
   const u32x4_t sHH = {h0, h1, h0, h1}, sL0 = {l0, l1, 0u, 0u};
   Y = mfma(o.Br, sHH, Y);
   Y = mfma(o.Br, sL0, Y);                     // Y^T += Mbr^T SA^T
+  if (next != nullptr) o.Br = *reinterpret_cast<const u32x4_t*>(&next->Mt[2][lane]);
   // state snapshot for `length` (one chunk per sequence)
   if (is_snap) {
     const bool keep = slot->keep_snap != 0;
@@ -508,7 +522,7 @@ __device__ __forceinline__ void consume(Consumer& C, const Ops& o, const Slot* _
       const u32x4_t sk = *reinterpret_cast<const u32x4_t*>(&snapslot->BT[1][tile][lane]);
       f32x4_t acc = keep ? C.S[tile] : zero4;
       acc = mfma(sb, sHH, acc);
-      acc = mfma(sk, o.vv, acc);
+      acc = mfma(sk, vv, acc);
       acc = mfma(sb, sL0, acc);
       const float4 sg = *reinterpret_cast<const float4*>(&snapslot->gamma[16 * tile + 4 * g]);
       acc[0] *= sg.x; acc[1] *= sg.y; acc[2] *= sg.z; acc[3] *= sg.w;
@@ -523,7 +537,7 @@ __device__ __forceinline__ void consume(Consumer& C, const Ops& o, const Slot* _
     }
   }
   // state update, tile by tile: rows = keys.  S <- (S + Bh^T SA^T + Kh^T V^T) . gamma
-  if (__builtin_amdgcn_readfirstlane(o.keep_end) == 0) {
+  if (!keep_end) {
     asm volatile("" ::: "memory");   // keep this a (rare, uniform) branch instead of 16 selects on the hot path
 #pragma unroll
     for (int tile = 0; tile < 4; ++tile) C.S[tile] = zero4;   // a reset inside the chunk cuts the entering state off
@@ -532,12 +546,11 @@ __device__ __forceinline__ void consume(Consumer& C, const Ops& o, const Slot* _
   for (int tile = 0; tile < 4; ++tile) {
     f32x4_t acc = C.S[tile];
     acc = mfma(bt[0][tile], sHH, acc);
-    acc = mfma(bt[1][tile], o.vv, acc);
+    acc = mfma(bt[1][tile], vv, acc);
     acc = mfma(bt[0][tile], sL0, acc);
     acc[0] *= gm[tile].x; acc[1] *= gm[tile].y; acc[2] *= gm[tile].z; acc[3] *= gm[tile].w;
     C.S[tile] = acc;
   }
-  prefetch();
   // outputs: register i is token 4g+i, lanes n = 16 consecutive values
   const uint32_t y01 = pack_rn(Y[0], Y[1]), y23 = pack_rn(Y[2], Y[3]);
   char* const yl = oc.y + (size_t)oc.voff * 2;
@@ -631,28 +644,19 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_fwd_kernel(Wk
     oc.voff = (uint32_t)((4 * (lane >> 4)) * (int)A.H * 64 + 16 * wave + (lane & 15));
     const int csnap = L >= 1 ? (int)((L - 1) / CK) : -1;
     const int nch = (int)nchunks;
-    // one chunk: consume with operand set `cur`, fetching the next chunk's set into `nxt` on the way
-    auto step = [&](int c, const Ops& cur, Ops& nxt) {
-      const int nvalid = (c + 1 < nch || A.T % CK == 0) ? CK : (int)(A.T % CK);
-      const int si = c % RING;
-      consume(C, cur, &slots[si], snapslot, A, b, h, nvalid, c == csnap, q2drop, oc, [&]() {
-        if (c + 1 < nch) {
-          const int sn = (c + 1) % RING;
-          wait_ready(sy, sn, c + 2);
-          load_ops(nxt, &slots[sn], wave, lane);
-        }
-      });
-      // every LDS read of slot si has returned: its data went into the MFMAs above
-      if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], c + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
-    };
-    Ops opA, opB;
+    Ops ops;
     if (nch > 0) {
       wait_ready(sy, 0, 1);
-      load_ops(opA, &slots[0], wave, lane);
+      load_ops(ops, &slots[0], wave, lane);
     }
-    for (int c = 0; c < nch; c += 2) {
-      step(c, opA, opB);
-      if (c + 1 < nch) step(c + 1, opB, opA);
+    for (int c = 0; c < nch; ++c) {
+      const int nvalid = (c + 1 < nch || A.T % CK == 0) ? CK : (int)(A.T % CK);
+      const int si = c % RING, sn = (c + 1) % RING;
+      const Slot* next = (c + 1 < nch) ? &slots[sn] : nullptr;
+      consume(C, ops, &slots[si], next, snapslot, A, b, h, nvalid, c == csnap, q2drop, oc,
+              [&]() { wait_ready(sy, sn, c + 2); });
+      // every LDS read of slot si has returned: its data went into the MFMAs above
+      if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], c + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
   } else {
     const int p = wave - NCONS;
