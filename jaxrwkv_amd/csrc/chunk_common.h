@@ -1,0 +1,139 @@
+// Building blocks shared by the chunked MFMA kernels (gfx950): bf16 hi/lo operand splitting, the 16x16x32 bf16
+// MFMA wrapper, DPP helpers for the in-chunk decay scan, per-chunk reset/length facts, and the LDS hand-shake
+// between producer and consumer waves.
+#pragma once
+#include "common.h"
+
+namespace hiprwkv {
+namespace chunk {
+
+typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+constexpr int CK = 16;            // tokens per chunk
+constexpr int RS = 72;            // row stride (bf16 elements) of the [token][64] LDS arrays: 144 B (16-byte aligned rows)
+constexpr int NCONS = 4;          // consumer waves, one per 16 value rows
+constexpr int SPIN_LIMIT = 1 << 16;   // polls before a waiter gives up (milliseconds; a healthy wait is microseconds)
+constexpr float LOG2E = 1.44269504088896340736f;
+constexpr float MIN_STEP_L2 = -1.0e4f;          // keeps the running sum finite
+constexpr float MIN_CUM_L2 = -80.0f * LOG2E;    // 2^MIN_CUM_L2 = e^-80
+
+// Hand-shake words.  ready[s] = c + 1 once chunk c is complete in slot s; consumed[q][s] = c + 1 once consumer
+// q no longer reads chunk c in slot s.  Waiting is a bounded poll, so that a broken hand-shake ends the kernel
+// (with wrong results) instead of hanging the GPU.
+struct __attribute__((aligned(16))) Sync {
+  int ready[8];
+  int consumed[NCONS][8];
+};
+
+__device__ __forceinline__ void wait_ready(const Sync* sy, int slot, int want) {
+  for (int spin = 0; spin < SPIN_LIMIT; ++spin) {
+    if (__hip_atomic_load(&sy->ready[slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) == want) return;
+    __builtin_amdgcn_s_sleep(1);
+  }
+}
+__device__ __forceinline__ void wait_consumed(const Sync* sy, int slot, int want, int lane) {
+  for (int spin = 0; spin < SPIN_LIMIT; ++spin) {
+    int seen = want;
+    if (lane < NCONS) seen = __hip_atomic_load(&sy->consumed[lane][slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (__ballot(seen < want) == 0ull) return;
+    __builtin_amdgcn_s_sleep(1);
+  }
+}
+
+__device__ __forceinline__ f32x4_t mfma(const u32x4_t a, const u32x4_t b, f32x4_t c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+}
+
+__device__ __forceinline__ uint32_t pack_rn(float x0, float x1) {
+  bf16x2_t p = {(__bf16)x0, (__bf16)x1};
+  return __builtin_bit_cast(uint32_t, p);
+}
+// both values are exactly representable in bf16: keep the high halves
+__device__ __forceinline__ uint32_t pack_exact(float x0, float x1) {
+  return __builtin_amdgcn_perm(__float_as_uint(x1), __float_as_uint(x0), 0x07060302u);
+}
+
+// (x0, x1) -> packed truncated-bf16 hi parts and packed bf16 lo parts (x = hi + lo up to 2^-17 relative)
+__device__ __forceinline__ void split2(float x0, float x1, uint32_t& hi, uint32_t& lo) {
+  hi = __builtin_amdgcn_perm(__float_as_uint(x1), __float_as_uint(x0), 0x07060302u);
+  // x - hi in one v_dot2c_f32_bf16 each: acc += hi.lo * -1 + hi.hi * 0  (resp. 0, -1)
+  // The two selectors are kept out of the compiler's sight: written as immediates, (-1, 0) would be encoded as
+  // the 16-bit inline constant -1.0, whose bit pattern is the fp16 one.
+  const bf16x2_t hp = __builtin_bit_cast(bf16x2_t, hi);
+  uint32_t m10 = 0x0000bf80u, m01 = 0xbf800000u;
+  asm volatile("" : "+s"(m10), "+s"(m01));
+  const float l0 = __builtin_amdgcn_fdot2_f32_bf16(hp, __builtin_bit_cast(bf16x2_t, m10), x0, false);
+  const float l1 = __builtin_amdgcn_fdot2_f32_bf16(hp, __builtin_bit_cast(bf16x2_t, m01), x1, false);
+  lo = pack_rn(l0, l1);
+}
+
+template <int CTRL>
+__device__ __forceinline__ float dpp0(float x) {  // lanes without a source read 0
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// inclusive sum over the 16 lanes of a DPP row
+__device__ __forceinline__ float row_scan(float x) {
+  x += dpp0<0x111>(x);
+  x += dpp0<0x112>(x);
+  x += dpp0<0x114>(x);
+  x += dpp0<0x118>(x);
+  return x;
+}
+// value of the previous lane of the row; `first` in lane 0 of the row
+__device__ __forceinline__ float row_prev(float x, float first) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(first), __float_as_int(x), 0x111, 0xf, 0xf, false));
+}
+
+__device__ __forceinline__ void unpack8(const uint4 p, float (&o)[8]) {
+  const uint32_t w[4] = {p.x, p.y, p.z, p.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    o[2 * i] = __uint_as_float(w[i] << 16);
+    o[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+  }
+}
+
+// Per-chunk facts, identical in every lane.
+struct ChunkFlags {
+  uint32_t ns;      // bit t: new_starts[c0+t], bit 16: new_starts[c0+16] (0 beyond T)
+  int nvalid;       // tokens of this chunk that exist
+  int snap;         // in-chunk index of token length-1, or -1
+  bool compat;
+};
+
+// number of resets at or before in-chunk token t: the index of its segment
+__device__ __forceinline__ int seg_of(uint32_t ns, int t) { return __builtin_popcount(ns & ((2u << t) - 1u)); }
+
+__device__ __forceinline__ ChunkFlags chunk_flags(const uint8_t* ns, unsigned flags, int64_t T, int64_t b, int64_t c0,
+                                                  int64_t L, int lane) {
+  ChunkFlags F;
+  F.compat = (flags & 1u) != 0;
+  F.nvalid = (int)((T - c0 < CK) ? (T - c0) : CK);
+  F.snap = (L >= 1 && L - 1 >= c0 && L - 1 < c0 + CK) ? (int)(L - 1 - c0) : -1;
+  // lanes 0..16 fetch one flag each; the ballot makes the 17-bit mask uniform
+  bool mine = false;
+  if (ns != nullptr && lane <= CK && c0 + lane < T) mine = ns[(size_t)b * T + c0 + lane] != 0;
+  F.ns = (uint32_t)(__ballot(mine) & 0x1ffffull);
+  return F;
+}
+
+// Selection operands that turn an MFMA into a transposer: against an A operand whose k-slot (g, jj) stands for key
+// 8g + jj of a 32-key half, B = sel[x] yields D[token][n] = value at key 16x + n.
+__device__ __forceinline__ void make_sel(u32x4_t (&sel)[2], int lane) {
+  const int n = lane & 15, g = lane >> 4;
+#pragma unroll
+  for (int x = 0; x < 2; ++x) {
+    const int jj = 16 * x + n - 8 * g;
+    u32x4_t sl = {0u, 0u, 0u, 0u};
+    if (jj >= 0 && jj < 8) sl[jj >> 1] = (jj & 1) ? 0x3f800000u : 0x00003f80u;
+    sel[x] = sl;
+  }
+}
+
+}  // namespace chunk
+}  // namespace hiprwkv

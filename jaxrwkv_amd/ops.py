@@ -120,8 +120,10 @@ def wkv7(r, w, k, v, a, b, s, length=None, new_starts=None, compat=True):
 
 
 # ----------------------------------------------------------------------------- WKV6
-def wkv6_fwd(r, k, v, w, u, s, length=None, new_starts=None, compat=True):
-    """r,k,v,w (B,T,H,N); u (H,N); s (B,H,N,N) [key, value].  Returns (new_s, y)."""
+def wkv6_fwd(r, k, v, w, u, s, length=None, new_starts=None, compat=True, force_seq=False):
+    """r,k,v,w (B,T,H,N); u (H,N); s (B,H,N,N) [key, value].  Returns (new_s, y).
+
+    bf16 inputs run on the chunked MFMA kernel unless ``force_seq`` asks for the sequential fp32 one."""
     lib = _lib.load()
     io = r.dtype
     B, T, H, N = r.shape
@@ -133,7 +135,8 @@ def wkv6_fwd(r, k, v, w, u, s, length=None, new_starts=None, compat=True):
     y = torch.empty_like(r)
     new_s = torch.empty_like(s)
     rc = lib.hiprwkv_wkv6_fwd(_stream(), _DT[io], _DT[s.dtype], B, T, H, N, _p(r), _p(k), _p(v), _p(w), _p(u), _p(s),
-                              _p(length), _p(new_starts), _p(y), _p(new_s), _flags(compat))
+                              _p(length), _p(new_starts), _p(y), _p(new_s),
+                              _flags(compat, force_seq))
     _lib.check(rc, "hiprwkv_wkv6_fwd")
     return new_s, y
 
