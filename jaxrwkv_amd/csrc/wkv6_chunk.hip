@@ -81,7 +81,7 @@ __device__ __forceinline__ void load_raw(Raw& x, const Wkv6Args& A, int64_t b, i
 struct Producer {
   int lane;
   u32x4_t sel[2];     // MFMA-as-transposer selection operands
-  uint4 u[2];         // the bonus of this lane's keys (bf16)
+  const char* u;      // the bonus of this lane's keys (bf16): 16 bytes here and 16 bytes 64 bytes further on
 };
 
 __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const ChunkFlags& F, Slot* __restrict__ slot,
@@ -151,7 +151,8 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
     u32x4_t qt_h, qt_l, kh_h, kh_l;
     {
       float fr[8], fk[8], fu[8], Einv[8], Ee[8];
-      unpack8(x.r[hf], fr); unpack8(x.k[hf], fk); unpack8(P.u[hf], fu);
+      unpack8(x.r[hf], fr); unpack8(x.k[hf], fk);
+      unpack8(*reinterpret_cast<const uint4*>(P.u + 64 * hf), fu);   // re-read per chunk (cache hit): frees registers
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const float l2 = fmaxf(E[e], MIN_CUM_L2);
@@ -277,12 +278,8 @@ __device__ __forceinline__ void consume(Consumer& C, Ops& o, const Slot* __restr
   const int lane = C.lane, n = lane & 15, g = lane >> 4;
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
   u32x4_t kt[4];
-  float4 gm[4];
 #pragma unroll
-  for (int tile = 0; tile < 4; ++tile) {
-    kt[tile] = *reinterpret_cast<const u32x4_t*>(&slot->KT[tile][lane]);
-    gm[tile] = *reinterpret_cast<const float4*>(&slot->gamma[16 * tile + 4 * g]);
-  }
+  for (int tile = 0; tile < 4; ++tile) kt[tile] = *reinterpret_cast<const u32x4_t*>(&slot->KT[tile][lane]);
   const bool keep_end = __builtin_amdgcn_readfirstlane(o.keep_end) != 0;
   // B operands from the state: MFMA j contracts over the keys of tiles 2j and 2j+1
   u32x4_t Sh[2], Sl[2];
@@ -302,6 +299,11 @@ __device__ __forceinline__ void consume(Consumer& C, Ops& o, const Slot* __restr
     Y = mfma(o.qt[1][j], Sh[j], Y);
   }
   const u32x4_t vv = o.vv;
+  // Qt and the Gram tile are dead now: fetch the next chunk's into the same registers, and this chunk's decay
+  asm volatile("" ::: "memory");   // keeps these loads below the products above (register pressure)
+  float4 gm[4];
+#pragma unroll
+  for (int tile = 0; tile < 4; ++tile) gm[tile] = *reinterpret_cast<const float4*>(&slot->gamma[16 * tile + 4 * g]);
   if (next != nullptr) {
     next_ready();
     load_ops(o, next, C.q, lane);
@@ -309,6 +311,10 @@ __device__ __forceinline__ void consume(Consumer& C, Ops& o, const Slot* __restr
   // state snapshot for `length` (one chunk per sequence)
   if (is_snap) {
     const bool keep = slot->keep_snap != 0;
+    // lane part of the state address, formed here so that it does not stay live across the chunk loop
+    uint32_t lane_el = (uint32_t)(4 * g * 64 + 16 * C.q + n);
+    asm volatile("" : "+v"(lane_el));
+    char* const base = reinterpret_cast<char*>(A.new_s) + state_off(A, b, h, 0, 0) * (A.st_f32 ? 4 : 2);
 #pragma unroll
     for (int tile = 0; tile < 4; ++tile) {
       const u32x4_t sk = *reinterpret_cast<const u32x4_t*>(&snapslot->KT[tile][lane]);
@@ -317,10 +323,10 @@ __device__ __forceinline__ void consume(Consumer& C, Ops& o, const Slot* __restr
       acc[0] *= sg.x; acc[1] *= sg.y; acc[2] *= sg.z; acc[3] *= sg.w;
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const size_t off = state_off(A, b, h, 16 * tile + 4 * g + i, 16 * C.q + n);
+        const uint32_t el = lane_el + (uint32_t)((16 * tile + i) * 64);
         const float x = q2drop ? 0.f : acc[i];
-        if (A.st_f32) reinterpret_cast<float*>(A.new_s)[off] = x;
-        else reinterpret_cast<uint16_t*>(A.new_s)[off] = f32_to_bf16(x);
+        if (A.st_f32) *reinterpret_cast<float*>(base + (size_t)el * 4) = x;
+        else *reinterpret_cast<uint16_t*>(base + (size_t)el * 2) = f32_to_bf16(x);
       }
     }
   }
@@ -387,7 +393,7 @@ __device__ __forceinline__ void store_state0(const Consumer& C, const Wkv6Args& 
 // Slot c % RING holds chunk c.  Producer p fills it once every consumer has released chunk c - RING, then
 // publishes ready = c + 1; consumers take chunks in order.  Every wait is for a strictly earlier chunk, so the
 // hand-shake cannot cycle.
-__global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv6_chunk_fwd_kernel(Wkv6Args A) {
+__global__ __launch_bounds__(64 * (NCONS + NPROD), 4) void wkv6_chunk_fwd_kernel(Wkv6Args A) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   Slot* slots = reinterpret_cast<Slot*>(smem_raw);
   SnapSlot* snapslot = reinterpret_cast<SnapSlot*>(smem_raw + RING * sizeof(Slot));
@@ -434,11 +440,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv6_chunk_fwd_kernel(Wk
     Producer P;
     P.lane = lane;
     make_sel(P.sel, lane);
-    {
-      const char* up = reinterpret_cast<const char*>(A.u) + ((size_t)h * 64 + 8 * (lane >> 4)) * 2;
-      P.u[0] = *reinterpret_cast<const uint4*>(up);
-      P.u[1] = *reinterpret_cast<const uint4*>(up + 64);
-    }
+    P.u = reinterpret_cast<const char*>(A.u) + ((size_t)h * 64 + 8 * (lane >> 4)) * 2;
     Raw raw;
     if (p < nchunks) load_raw(raw, A, b, h, (int64_t)p * CK, lane);
     for (int64_t c = p; c < nchunks; c += NPROD) {

@@ -1,6 +1,7 @@
-// WKV7 forward, chunked MFMA kernel for bf16 I/O on gfx950.
+// WKV7 chunked MFMA kernels for bf16 I/O on gfx950: the forward pass and the first (reverse) sweep of the backward.
 //
-// Recurrence per head (reference: /root/reference/src/jaxrwkv/rwkv7.py:200-220), S[i][j] = value row i, key col j:
+// Forward.  Recurrence per head (reference: /root/reference/src/jaxrwkv/rwkv7.py:200-220), S[i][j] = value row i,
+// key col j:
 //     sa_t = S_{t-1} a_t ;  S_t = S_{t-1} diag(d_t) + sa_t b_t^T + v_t k_t^T ;  y_t = S_t r_t ;  d_t = exp(-exp(w_t))
 // A chunk of C = 16 tokens entering with state S0 is evaluated in closed form.  With l_t = log d_t,
 // Lc_t = sum_{s<=t} l_s, E_t = exp(Lc_t), Ee_t = exp(Lc_{t-1}) and the scaled operands
@@ -17,20 +18,30 @@
 // MFMA hold two 16-token products side by side.  The state stays in fp32 accumulator registers for the whole
 // sequence, transposed (key x value tiles), so that accumulator registers are reused directly as B operands.
 //
+// Reverse sweep (REV).  With G = dL/dS carried from the last token down (G~_t the cotangent of S_t):
+//     G~_t = dy_t r_t^T + G~_{t+1} diag(d_{t+1}) + dsa_{t+1} a_{t+1}^T ;  dsa_t = G~_t b_t ;  dv_t = G~_t k_t
+// Inside a chunk leaving with G_C (cotangent of the chunk-end state from later chunks), Gh = G_C diag(E_C):
+//     G~_t diag(E_t) = Gh + sum_{s>=t} dy_s qt_s^T + sum_{s>t} dsa_s at_s^T
+//     U   = Gh Bh^T + DY^T Mbr^T         DSA = U (I - Mba^T)^{-1}         DV = Gh Kh^T + DSA Mka^T + DY^T Mkr^T
+//     G_prev = Gh + DSA At + DY^T Qt      (cotangent of the state entering the chunk)
+// which is the forward computation with the operands exchanged (Bh <-> At, Kh <-> Qt, V <-> DY, every Gram tile
+// transposed) and the decay applied before instead of after the update; the same code runs both.
+//
 // Work split: one workgroup of 8 waves per (sequence, head).  Waves 0-3 are consumers: wave q owns value rows
-// 16q..16q+15 of the state and runs the S0-dependent part of every chunk.  Waves 4-7 are producers: producer p
-// prepares chunks p, p+4, p+8, ... (everything that does not depend on S0: decay scan, scaled operands, Gram
-// tiles, triangular inverse, operand transposes) into a ring of LDS slots, four chunk periods ahead of the
+// 16q..16q+15 of the state and runs the state-dependent part of every chunk.  Waves 4-7 are producers: producer p
+// prepares chunks p, p+4, p+8, ... (everything that does not depend on the state: decay scan, scaled operands,
+// Gram tiles, triangular inverse, operand transposes) into a ring of LDS slots, four chunk periods ahead of the
 // consumers.  Synchronisation is a pair of LDS sequence numbers per slot: `ready` (set by the producer when a
 // chunk is complete) and `consumed` (one per consumer wave, set when it has read the slot for the last time).
 // Waiting is a bounded poll, so that a broken hand-shake ends the kernel (with wrong results) instead of
 // hanging the GPU.
 // new_starts inside a chunk restart the cumulative decay and mask the Gram tiles (rare, uniform branch).
-// `length` snapshots use a second, masked set of update operands for the one chunk that holds token length-1.
+// The one chunk that holds token length-1 uses a second, masked operand set: for the state snapshot in the
+// forward pass, for the entry of the returned state's cotangent in the reverse sweep.
 //
 // Range: the cumulative log decay inside a chunk is clamped at -80 so that 1/E_s stays finite in fp32.  A key
 // channel whose decay over at most 16 tokens falls below e^-80 (RWKV-7 models keep d >= 0.54 per token, i.e.
-// e^-10 per chunk) is finite but no longer exact; the sequential kernel has no such limit.
+// e^-10 per chunk) is finite but no longer exact; the sequential kernels have no such limit.
 #include "chunk_common.h"
 #include "wkv_args.h"
 
@@ -47,6 +58,8 @@ constexpr int RING = 5;           // slots in flight
 // the 16 bytes that the same lane of a consumer loads: accumulator-layout registers (column lane%16, rows
 // 4*(lane/16)..+3) packed to bf16, hi pair then lo pair, which is exactly an A operand (row lane%16, k-slots
 // 4*(lane/16)..+3 of the hi part followed by the same slots of the lo part).
+// Names are the forward ones; the reverse sweep stores (Bh, Kh) rows in AQ, (at, qt)^T in BT, dy^T in VT and the
+// transposed Gram tiles (inverse, Mbr^T, Mka^T, Mkr^T) in Mt.
 struct __attribute__((aligned(16))) Slot {
   // At = a_t.Ee_t and Qt = r_t.E_t, [hi|lo][At|Qt][token][RS]: within a row, the 16-byte vector (j, g) at element
   // 32j + 8g holds keys 32j+4g..+3 followed by keys 32j+16+4g..+3, the key order of the consumers' state tiles.
@@ -57,22 +70,31 @@ struct __attribute__((aligned(16))) Slot {
   uint4 Mt[4][64];             // T, Mka, Mbr, Mkr: hi,lo, lane-indexed
   float gamma[64];             // E at the chunk end
   int snap;                    // -1, or the in-chunk index of token length-1
-  int keep_end;                // the entering state survives to the chunk end (no reset in the chunk)
-  int keep_snap;               // the entering state survives to the snapshot token
+  int keep_end;                // the carried state passes through the whole chunk (no reset in the chunk)
+  int keep_snap;               // forward: the entering state survives to the snapshot token;
+                               // reverse: the cotangent entering at token length-1 reaches the chunk start
   int pad;
 };
-// Update operands masked for the snapshot token; only one chunk per sequence needs them.
-struct __attribute__((aligned(16))) SnapSlot {
+// Operands masked for token length-1; only one chunk per sequence needs them.  Forward: update operands for the
+// state snapshot.  Reverse: row operands for the cotangent of the returned state.
+template <bool REV> struct SnapSlotT;
+template <> struct __attribute__((aligned(16))) SnapSlotT<false> {
   uint4 BT[2][4][64];
   float gamma[64];
 };
+template <> struct __attribute__((aligned(16))) SnapSlotT<true> {
+  uint16_t AQ[2][2][CK][RS];
+  float gamma[64];
+};
+
 // ---------------------------------------------------------------------------------------------------- producer
 // Lane (t = lane%16, g = lane/16) owns token t and the keys {8g..8g+7} u {32+8g..32+8g+7}: exactly the A/B
 // operand layout of the Gram MFMAs (row/column = token, k-slots = keys), and one 16-byte global load per half.
 struct Raw {
-  uint4 r[2], w[2], k[2], v[2], a[2], b[2];
+  uint4 r[2], w[2], k[2], v[2], a[2], b[2];   // v holds dy in the reverse sweep
 };
 
+template <bool REV>
 __device__ __forceinline__ void load_raw(Raw& x, const Wkv7Args& A, int64_t b, int64_t h, int64_t c0, int lane) {
   const int t = lane & 15, g = lane >> 4;
   const uint4 z = make_uint4(0, 0, 0, 0);
@@ -82,7 +104,7 @@ __device__ __forceinline__ void load_raw(Raw& x, const Wkv7Args& A, int64_t b, i
       o[0] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(p) + off);
       o[1] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(p) + off + 64);
     };
-    ld(A.r, x.r); ld(A.w, x.w); ld(A.k, x.k); ld(A.v, x.v); ld(A.a, x.a); ld(A.b, x.b);
+    ld(A.r, x.r); ld(A.w, x.w); ld(A.k, x.k); ld(REV ? A.gy : A.v, x.v); ld(A.a, x.a); ld(A.b, x.b);
   } else {
     x.r[0] = x.r[1] = x.w[0] = x.w[1] = x.k[0] = x.k[1] = z;
     x.v[0] = x.v[1] = x.a[0] = x.a[1] = x.b[0] = x.b[1] = z;
@@ -94,35 +116,42 @@ struct Producer {
   u32x4_t sel[2];     // B operands that pick keys 16*(tile%2)..+15 out of a 32-key half: MFMA as a transposer
 };
 
-// Everything of one chunk that does not depend on the entering state.  The two 32-key halves go through the
+// Everything of one chunk that does not depend on the carried state.  The two 32-key halves go through the
 // same pipeline one after the other (scan, scaling, hi/lo split, LDS parking, transposes, partial Gram sums),
-// which keeps the live register set small enough for three waves per SIMD.
+// which keeps the live register set small.
+template <bool REV>
 __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const ChunkFlags& F, Slot* __restrict__ slot,
-                                        SnapSlot* __restrict__ snap) {
+                                        SnapSlotT<REV>* __restrict__ snap) {
   const int lane = P.lane, t = lane & 15, g = lane >> 4;
   const bool valid = t < F.nvalid;
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
-  const u32x4_t z4 = {0u, 0u, 0u, 0u};
   const bool slow = F.ns != 0;                    // a reset in this chunk or at the first token of the next
   const uint32_t resets = F.ns & 0xffffu;
   // reset bookkeeping (uniform values unless they depend on t)
   int lastseg = 0, seg_src = 0;
-  bool s0_reaches = true, q_keep = true, restart = false, at_reset = false;
+  bool row0_keep = true, row1_keep = true, restart = false, at_reset = false, drop_dy = false;
   uint32_t keep_upd = 0xffffu, keep_snap = 0;
   if (F.snap >= 0) keep_snap = (2u << F.snap) - 1u;
   if (slow) {
     lastseg = seg_of(F.ns, 15);
-    s0_reaches = seg_of(F.ns, t) == 0;                              // the entering state reaches this token
-    q_keep = s0_reaches && !(F.compat && ((F.ns >> (t + 1)) & 1u)); // y[t] is defined as zero before a reset
-    if (resets) keep_upd = 0xffffu & ~((1u << (31 - __builtin_clz(resets))) - 1u);   // tokens from the last reset on
+    const int myseg = seg_of(F.ns, t);
+    if (!REV) {
+      row0_keep = myseg == 0;                                          // the entering state reaches this token
+      row1_keep = row0_keep && !(F.compat && ((F.ns >> (t + 1)) & 1u)); // y[t] is defined as zero before a reset
+      if (resets) keep_upd = 0xffffu & ~((1u << (31 - __builtin_clz(resets))) - 1u);   // tokens from the last reset on
+      at_reset = (resets >> t) & 1u;
+    } else {
+      row0_keep = row1_keep = myseg == lastseg;                        // the cotangent from later chunks reaches this token
+      if (resets) keep_upd = (1u << __builtin_ctz(resets)) - 1u;       // tokens before the first reset
+      drop_dy = F.compat && ((F.ns >> (t + 1)) & 1u);                  // y[t] is a constant there
+    }
     const uint32_t upto = resets & ((2u << t) - 1u);
     const int pr = upto ? 31 - __builtin_clz(upto) : 0;             // last reset at or before this token
     restart = pr > 0;
     seg_src = (lane & 48) | (pr > 0 ? pr - 1 : 0);
-    at_reset = (resets >> t) & 1u;
     if (F.snap >= 0) {
       const uint32_t us = resets & keep_snap;
-      if (us) keep_snap &= ~((1u << (31 - __builtin_clz(us))) - 1u);
+      if (us) keep_snap &= ~((1u << (31 - __builtin_clz(us))) - 1u);   // tokens of length-1's segment up to it
     }
   }
   auto masked_pack = [&](const f32x4_t d, uint32_t keep) {
@@ -134,12 +163,15 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
   auto plain_pack = [&](const f32x4_t d) { return make_uint2(pack_exact(d[0], d[1]), pack_exact(d[2], d[3])); };
   auto join = [&](const uint2 hi, const uint2 lo) { return make_uint4(hi.x, hi.y, lo.x, lo.y); };
 
-  f32x4_t Mba = zero4, MbaT = zero4, Mka = zero4, Mbr = zero4, Mkr = zero4;
+  // Gram tiles in accumulator layout [row m = A-operand token][column n = B-operand token]
+  f32x4_t Gab = zero4, GabT = zero4;   // bh_m.at_n and at_m.bh_n
+  f32x4_t G1 = zero4, G2 = zero4, G3 = zero4;   // forward: Mka, Mbr, Mkr; reverse: qt_m.bh_n, at_m.kh_n, qt_m.kh_n
 #pragma unroll
   for (int hf = 0; hf < 2; ++hf) {
-    // ---- v^T of value tiles 2hf, 2hf+1: D[token][value] = sum_k V[token][k] sel[k][value]
+    // ---- v^T (dy^T) of value tiles 2hf, 2hf+1: D[token][value] = sum_k V[token][k] sel[k][value]
     {
-      const uint4 vr = x.v[hf];
+      uint4 vr = x.v[hf];
+      if (REV && drop_dy) vr = make_uint4(0, 0, 0, 0);
       const u32x4_t vop = {vr.x, vr.y, vr.z, vr.w};
 #pragma unroll
       for (int x2 = 0; x2 < 2; ++x2) slot->VT[2 * hf + x2][lane] = plain_pack(mfma(vop, P.sel[x2], zero4));
@@ -153,11 +185,7 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
       for (int e = 0; e < 8; ++e) {
         float l2 = fmaxf(-exp2_fast(fw[e] * LOG2E) * LOG2E, MIN_STEP_L2);
         if (F.nvalid != CK) l2 = valid ? l2 : 0.f;
-        l2 += dpp0<0x111>(l2);
-        l2 += dpp0<0x112>(l2);
-        l2 += dpp0<0x114>(l2);
-        l2 += dpp0<0x118>(l2);
-        E[e] = l2;
+        E[e] = row_scan(l2);
       }
     }
     unpack8(x.a[hf], fa);
@@ -166,7 +194,7 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
       for (int e = 0; e < 8; ++e) {
         const float base = __shfl(E[e], seg_src, 64);   // restart the cumulative decay at the last reset
         if (restart) E[e] -= base;
-        if (at_reset) fa[e] = 0.f;                      // the state entering a reset token is zero: sa = 0
+        if (!REV && at_reset) fa[e] = 0.f;              // the state entering a reset token is zero: sa = 0
       }
     }
     // ---- scaled operands and their hi/lo split
@@ -179,8 +207,9 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
         const float l2 = fmaxf(E[e], MIN_CUM_L2);
         E[e] = exp2_fast(l2);
         Einv[e] = exp2_fast(-l2);
-        // exclusive: value of the previous token; 1 for the first token of the chunk (a is zero at reset tokens)
-        Ee[e] = __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(1.0f), __float_as_int(E[e]), 0x111, 0xf, 0xf, false));
+        // exclusive: value of the previous token; 1 for the first token of the chunk.  At a reset token the value
+        // belongs to the previous segment, but every product it enters is masked out or multiplies a zero.
+        Ee[e] = row_prev(E[e], 1.0f);
       }
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -192,7 +221,7 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
         split2(fb[e] * Einv[e], fb[e + 1] * Einv[e + 1], hi, lo); bh_h[j] = hi; bh_l[j] = lo;
       }
     }
-    // ---- decay to the chunk end / to the snapshot token
+    // ---- decay to the chunk end / to token length-1
     if (t == 15) {
       float* gp = &slot->gamma[8 * g + 32 * hf];
       *reinterpret_cast<float4*>(gp) = make_float4(E[0], E[1], E[2], E[3]);
@@ -203,94 +232,118 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
       *reinterpret_cast<float4*>(gp) = make_float4(E[0], E[1], E[2], E[3]);
       *reinterpret_cast<float4*>(gp + 4) = make_float4(E[4], E[5], E[6], E[7]);
     }
-    // ---- At, Qt rows for the consumers, in their key order: this lane's keys 8g..8g+3 and 8g+4..8g+7 of the half
-    //      are the (g>>1)-th 8-byte piece of the vectors 2(g&1) and 2(g&1)+1 of block j = hf
+    // ---- row operands for the consumers (forward At, Qt; reverse Bh, Kh), in their key order: this lane's keys
+    //      8g..8g+3 and 8g+4..8g+7 of the half are the (g>>1)-th 8-byte piece of the vectors 2(g&1) and 2(g&1)+1
+    //      of block j = hf
     {
+      const u32x4_t &r0h = REV ? bh_h : at_h, &r0l = REV ? bh_l : at_l;
+      const u32x4_t &r1h = REV ? kh_h : qt_h, &r1l = REV ? kh_l : qt_l;
       const int e0 = 32 * hf + 16 * (g & 1) + 4 * (g >> 1);     // element offset of the first piece
       auto put = [&](uint16_t* row, const u32x4_t v, bool keep) {
         *reinterpret_cast<uint2*>(row + e0) = keep ? make_uint2(v[0], v[1]) : make_uint2(0u, 0u);
         *reinterpret_cast<uint2*>(row + e0 + 8) = keep ? make_uint2(v[2], v[3]) : make_uint2(0u, 0u);
       };
       if (!slow) {
-        put(slot->AQ[0][0][t], at_h, true); put(slot->AQ[1][0][t], at_l, true);
-        put(slot->AQ[0][1][t], qt_h, true); put(slot->AQ[1][1][t], qt_l, true);
+        put(slot->AQ[0][0][t], r0h, true); put(slot->AQ[1][0][t], r0l, true);
+        put(slot->AQ[0][1][t], r1h, true); put(slot->AQ[1][1][t], r1l, true);
       } else {
-        put(slot->AQ[0][0][t], at_h, s0_reaches); put(slot->AQ[1][0][t], at_l, s0_reaches);
-        put(slot->AQ[0][1][t], qt_h, q_keep); put(slot->AQ[1][1][t], qt_l, q_keep);
+        put(slot->AQ[0][0][t], r0h, row0_keep); put(slot->AQ[1][0][t], r0l, row0_keep);
+        put(slot->AQ[0][1][t], r1h, row1_keep); put(slot->AQ[1][1][t], r1l, row1_keep);
+      }
+      if constexpr (REV) {
+        if (F.snap >= 0) {
+          const bool sk = (keep_snap >> t) & 1u;
+          put(snap->AQ[0][0][t], r0h, sk); put(snap->AQ[1][0][t], r0l, sk);
+          put(snap->AQ[0][1][t], r1h, sk); put(snap->AQ[1][1][t], r1l, sk);
+        }
       }
     }
-    // ---- (b/E)^T, (k/E)^T of key tiles 2hf, 2hf+1 by MFMA: the accumulator layout of D (lane = key, registers =
-    //      4 consecutive tokens) is the A-operand layout of the state update
+    // ---- transposed update operands of key tiles 2hf, 2hf+1 by MFMA (forward (b/E)^T, (k/E)^T; reverse at^T,
+    //      qt^T): the accumulator layout of D (lane = key, registers = 4 consecutive tokens) is the A-operand
+    //      layout of the state update
+    {
+      const u32x4_t &t0h = REV ? at_h : bh_h, &t0l = REV ? at_l : bh_l;
+      const u32x4_t &t1h = REV ? qt_h : kh_h, &t1l = REV ? qt_l : kh_l;
 #pragma unroll
-    for (int x2 = 0; x2 < 2; ++x2) {
-      const int tile = 2 * hf + x2;
-      const u32x4_t sel = P.sel[x2];
-      const f32x4_t dbh = mfma(bh_h, sel, zero4), dbl = mfma(bh_l, sel, zero4);
-      const f32x4_t dkh = mfma(kh_h, sel, zero4), dkl = mfma(kh_l, sel, zero4);
-      if (keep_upd == 0xffffu) {
-        slot->BT[0][tile][lane] = join(plain_pack(dbh), plain_pack(dbl));
-        slot->BT[1][tile][lane] = join(plain_pack(dkh), plain_pack(dkl));
-      } else {
-        slot->BT[0][tile][lane] = join(masked_pack(dbh, keep_upd), masked_pack(dbl, keep_upd));
-        slot->BT[1][tile][lane] = join(masked_pack(dkh, keep_upd), masked_pack(dkl, keep_upd));
-      }
-      if (F.snap >= 0) {
-        snap->BT[0][tile][lane] = join(masked_pack(dbh, keep_snap), masked_pack(dbl, keep_snap));
-        snap->BT[1][tile][lane] = join(masked_pack(dkh, keep_snap), masked_pack(dkl, keep_snap));
+      for (int x2 = 0; x2 < 2; ++x2) {
+        const int tile = 2 * hf + x2;
+        const u32x4_t sel = P.sel[x2];
+        const f32x4_t d0h = mfma(t0h, sel, zero4), d0l = mfma(t0l, sel, zero4);
+        const f32x4_t d1h = mfma(t1h, sel, zero4), d1l = mfma(t1l, sel, zero4);
+        if (keep_upd == 0xffffu) {
+          slot->BT[0][tile][lane] = join(plain_pack(d0h), plain_pack(d0l));
+          slot->BT[1][tile][lane] = join(plain_pack(d1h), plain_pack(d1l));
+        } else {
+          slot->BT[0][tile][lane] = join(masked_pack(d0h, keep_upd), masked_pack(d0l, keep_upd));
+          slot->BT[1][tile][lane] = join(masked_pack(d1h, keep_upd), masked_pack(d1l, keep_upd));
+        }
+        if constexpr (!REV) {
+          if (F.snap >= 0) {
+            snap->BT[0][tile][lane] = join(masked_pack(d0h, keep_snap), masked_pack(d0l, keep_snap));
+            snap->BT[1][tile][lane] = join(masked_pack(d1h, keep_snap), masked_pack(d1l, keep_snap));
+          }
+        }
       }
     }
     // ---- partial Gram sums over this half's keys (accumulator layout: column n = lane%16, rows 4g..4g+3)
 #pragma unroll
     for (int part = 0; part < 3; ++part) {
-      const u32x4_t bA = part == 2 ? bh_l : bh_h, kA = part == 2 ? kh_l : kh_h, aA = part == 2 ? at_l : at_h;
-      const u32x4_t aB = part == 1 ? at_l : at_h, qB = part == 1 ? qt_l : qt_h, bB = part == 1 ? bh_l : bh_h;
-      Mba = mfma(bA, aB, Mba);     // [s][t] = bh_s . at_t
-      MbaT = mfma(aA, bB, MbaT);   // [t][s]
-      Mka = mfma(kA, aB, Mka);     // [s][t] = kh_s . at_t
-      Mbr = mfma(bA, qB, Mbr);     // [s][t] = bh_s . qt_t
-      Mkr = mfma(kA, qB, Mkr);     // [s][t] = kh_s . qt_t
+      const u32x4_t bA = part == 2 ? bh_l : bh_h, kA = part == 2 ? kh_l : kh_h;
+      const u32x4_t aA = part == 2 ? at_l : at_h, qA = part == 2 ? qt_l : qt_h;
+      const u32x4_t aB = part == 1 ? at_l : at_h, qB = part == 1 ? qt_l : qt_h;
+      const u32x4_t bB = part == 1 ? bh_l : bh_h, kB = part == 1 ? kh_l : kh_h;
+      Gab = mfma(bA, aB, Gab);      // [m][n] = bh_m . at_n
+      GabT = mfma(aA, bB, GabT);    // [m][n] = at_m . bh_n
+      if constexpr (!REV) {
+        G1 = mfma(kA, aB, G1);      // Mka[m][n] = kh_m . at_n
+        G2 = mfma(bA, qB, G2);      // Mbr[m][n] = bh_m . qt_n
+        G3 = mfma(kA, qB, G3);      // Mkr[m][n] = kh_m . qt_n
+      } else {
+        G1 = mfma(qA, bB, G1);      // Mbr^T[m][n] = qt_m . bh_n
+        G2 = mfma(aA, kB, G2);      // Mka^T[m][n] = at_m . kh_n
+        G3 = mfma(qA, kB, G3);      // Mkr^T[m][n] = qt_m . kh_n
+      }
     }
   }
-  // ---- triangular masks
+  // ---- triangular masks: forward keeps earlier rows m for column n, the reverse sweep later rows
   const int n = t;
-  if (!slow) {
+  {
+    const bool dropy = !REV && slow && F.compat && ((F.ns >> (n + 1)) & 1u);   // y[n] is defined as zero
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int m = 4 * g + i;
-      Mba[i] = (m < n) ? Mba[i] : 0.f;
-      Mka[i] = (m < n) ? Mka[i] : 0.f;
-      Mbr[i] = (m <= n) ? Mbr[i] : 0.f;
-      Mkr[i] = (m <= n) ? Mkr[i] : 0.f;
-      MbaT[i] = (m > n) ? MbaT[i] : 0.f;   // [t = m][s = n], s < t
-    }
-  } else {
-    const bool dropy = F.compat && ((F.ns >> (n + 1)) & 1u);   // y[n] is defined as zero
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int m = 4 * g + i;
-      const bool same = seg_of(F.ns, m) == seg_of(F.ns, n);
-      const bool lt = (m < n) && same, le = (m <= n) && same, gt = (m > n) && same;
-      Mba[i] = lt ? Mba[i] : 0.f;
-      Mka[i] = lt ? Mka[i] : 0.f;
-      Mbr[i] = (le && !dropy) ? Mbr[i] : 0.f;
-      Mkr[i] = (le && !dropy) ? Mkr[i] : 0.f;
-      MbaT[i] = gt ? MbaT[i] : 0.f;
+      bool lt = m < n, le = m <= n, gt = m > n, ge = m >= n;
+      if (slow) {
+        const bool same = seg_of(F.ns, m) == seg_of(F.ns, n);
+        lt = lt && same; le = le && same; gt = gt && same; ge = ge && same;
+      }
+      Gab[i] = lt ? Gab[i] : 0.f;
+      GabT[i] = gt ? GabT[i] : 0.f;
+      if constexpr (!REV) {
+        G1[i] = lt ? G1[i] : 0.f;
+        G2[i] = (le && !dropy) ? G2[i] : 0.f;
+        G3[i] = (le && !dropy) ? G3[i] : 0.f;
+      } else {
+        G1[i] = ge ? G1[i] : 0.f;
+        G2[i] = gt ? G2[i] : 0.f;
+        G3[i] = ge ? G3[i] : 0.f;
+      }
     }
   }
-  // ---- T = (I + M^8)(I + M^4)(I + M^2)(I + M), single-bf16 operands
+  // ---- (I - M)^{-1} = (I + M^8)(I + M^4)(I + M^2)(I + M) in single bf16; forward M = Mba, reverse M = Mba^T
   auto single = [&](const f32x4_t d) {
     u32x4_t o = {pack_rn(d[0], d[1]), pack_rn(d[2], d[3]), 0u, 0u};
     return o;
   };
-  f32x4_t Pm = Mba;
+  f32x4_t Mp = REV ? GabT : Gab, MpT = REV ? Gab : GabT;
+  f32x4_t Pm = Mp;
 #pragma unroll
   for (int i = 0; i < 4; ++i) Pm[i] += (4 * g + i == n) ? 1.f : 0.f;
-  f32x4_t Mp = Mba, MpT = MbaT;
 #pragma unroll
   for (int lvl = 0; lvl < 3; ++lvl) {
     const u32x4_t om = single(Mp), omt = single(MpT);
-    const f32x4_t M2T = mfma(om, omt, zero4);      // (M^2)^T[t][s]
-    if (lvl < 2) Mp = mfma(omt, om, zero4);        // (M^2)[s][t]: A rows from the transpose, B columns from M
+    const f32x4_t M2T = mfma(om, omt, zero4);      // (M^2)^T
+    if (lvl < 2) Mp = mfma(omt, om, zero4);        // M^2: A rows from the transpose, B columns from M
     MpT = M2T;
     Pm = mfma(single(MpT), single(Pm), Pm);        // P += M^(2^(lvl+1)) P
   }
@@ -300,7 +353,7 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
     split2(d[2], d[3], hi1, lo1);
     slot->Mt[which][lane] = make_uint4(hi0, hi1, lo0, lo1);
   };
-  park(0, Pm); park(1, Mka); park(2, Mbr); park(3, Mkr);
+  park(0, Pm); park(1, G1); park(2, G2); park(3, G3);
   if (lane == 0) {
     slot->snap = F.snap;
     slot->keep_end = (lastseg == 0) ? 1 : 0;
@@ -309,8 +362,8 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
 }
 
 // ---------------------------------------------------------------------------------------------------- consumer
-// Wave q holds S^T for value rows 16q..16q+15 as four 16x16 accumulator tiles: lane (n = lane%16, g = lane/16),
-// S[tile][i] = S[value 16q+n][key 16*tile + 4g + i].
+// Wave q holds S^T (G^T in the reverse sweep) for value rows 16q..16q+15 as four 16x16 accumulator tiles: lane
+// (n = lane%16, g = lane/16), S[tile][i] = S[value 16q+n][key 16*tile + 4g + i].
 struct Consumer {
   f32x4_t S[4];
   int q, lane;
@@ -347,19 +400,40 @@ __device__ __forceinline__ void load_ops(Ops& o, const Slot* __restrict__ slot, 
   o.Br = *reinterpret_cast<const u32x4_t*>(&slot->Mt[2][lane]);
 }
 
-// Uniform output cursors of a consumer, advanced by one chunk per call.
+// Uniform output cursors of a consumer, moved by one chunk per call.
 struct OutCursor {
-  char* y;             // A.out at (b, c0, h, 0)
-  char* sa;            // A.sa at the same place, or null
+  char* y;             // forward A.out, reverse A.gv, at (b, c0, h, 0)
+  char* sa;            // forward A.sa (or null), reverse A.dsa, at the same place
   size_t tok_bytes;    // bytes between consecutive tokens in y (twice that in sa)
   uint32_t voff;       // lane part of the address, in elements: (4g * H) * 64 + value
 };
 
-// The S0-dependent part of one chunk.  `next` is the slot of the following chunk (null after the last one);
-// `next_ready` waits until its producer has published it.
-template <class WaitNext>
+// element offset of this lane's four consecutive keys of a state tile
+__device__ __forceinline__ size_t state_off(const Wkv7Args& A, int64_t b, int64_t h, int q, int lane, int tile) {
+  return (((size_t)b * A.H + h) * 64 + 16 * q + (lane & 15)) * 64 + 16 * tile + 4 * (lane >> 4);
+}
+__device__ __forceinline__ f32x4_t load_state_tile(const void* p, int f32, size_t off) {
+  f32x4_t r;
+  if (f32) {
+    const float4 x = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p) + off);
+    r[0] = x.x; r[1] = x.y; r[2] = x.z; r[3] = x.w;
+  } else {
+    const uint2 x = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(p) + off);
+    r[0] = __uint_as_float(x.x << 16); r[1] = __uint_as_float(x.x & 0xffff0000u);
+    r[2] = __uint_as_float(x.y << 16); r[3] = __uint_as_float(x.y & 0xffff0000u);
+  }
+  return r;
+}
+__device__ __forceinline__ void store_state_tile(void* p, int f32, size_t off, const f32x4_t v) {
+  if (f32) *reinterpret_cast<float4*>(reinterpret_cast<float*>(p) + off) = make_float4(v[0], v[1], v[2], v[3]);
+  else *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(p) + off) = make_uint2(pack_rn(v[0], v[1]), pack_rn(v[2], v[3]));
+}
+
+// The state-dependent part of one chunk.  `next` is the slot of the chunk handled after this one (null after the
+// last one); `next_ready` waits until its producer has published it.
+template <bool REV, class WaitNext>
 __device__ __forceinline__ void consume(Consumer& C, Ops& o, const Slot* __restrict__ slot,
-                                        const Slot* __restrict__ next, const SnapSlot* __restrict__ snapslot,
+                                        const Slot* __restrict__ next, const SnapSlotT<REV>* __restrict__ snapslot,
                                         const Wkv7Args& A, int64_t b, int64_t h, int nvalid, bool is_snap, bool q2drop,
                                         OutCursor& oc, WaitNext&& next_ready) {
   const int lane = C.lane, n = lane & 15, g = lane >> 4;
@@ -374,6 +448,13 @@ __device__ __forceinline__ void consume(Consumer& C, Ops& o, const Slot* __restr
     gm[tile] = *reinterpret_cast<const float4*>(&slot->gamma[16 * tile + 4 * g]);
   }
   const bool keep_end = __builtin_amdgcn_readfirstlane(o.keep_end) != 0;
+  if constexpr (REV) {
+    // the cotangent of the chunk-end state, decayed over the chunk
+#pragma unroll
+    for (int tile = 0; tile < 4; ++tile) {
+      C.S[tile][0] *= gm[tile].x; C.S[tile][1] *= gm[tile].y; C.S[tile][2] *= gm[tile].z; C.S[tile][3] *= gm[tile].w;
+    }
+  }
   // B operands from the state: MFMA j contracts over the keys of tiles 2j and 2j+1
   u32x4_t Sh[2], Sl[2];
 #pragma unroll
@@ -394,6 +475,40 @@ __device__ __forceinline__ void consume(Consumer& C, Ops& o, const Slot* __restr
   W = mfma(o.Ka, o.vv, W);                    // W += Mka^T V^T (hi and lo parts side by side)
   Y = mfma(o.Kr, o.vv, Y);                    // Y += Mkr^T V^T
   const u32x4_t vv = o.vv;
+  if constexpr (REV) {
+    // a reset inside the chunk cuts the cotangent of later chunks off from the chunk start
+    if (!keep_end) {
+      asm volatile("" ::: "memory");
+#pragma unroll
+      for (int tile = 0; tile < 4; ++tile) C.S[tile] = zero4;
+    }
+    // the cotangent of the returned state enters at token length-1 (one chunk per sequence)
+    if (is_snap) {
+      const bool keep = slot->keep_snap != 0;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        u32x4_t gh, gl;
+#pragma unroll
+        for (int x2 = 0; x2 < 2; ++x2) {
+          const int tile = 2 * j + x2;
+          f32x4_t gs = load_state_tile(A.gs_out, A.st_f32, state_off(A, b, h, C.q, lane, tile));
+          const float4 sg = *reinterpret_cast<const float4*>(&snapslot->gamma[16 * tile + 4 * g]);
+          gs[0] *= sg.x; gs[1] *= sg.y; gs[2] *= sg.z; gs[3] *= sg.w;
+          if (keep) C.S[tile] += gs;
+          uint32_t hi, lo;
+          split2(gs[0], gs[1], hi, lo); gh[2 * x2] = hi; gl[2 * x2] = lo;
+          split2(gs[2], gs[3], hi, lo); gh[2 * x2 + 1] = hi; gl[2 * x2 + 1] = lo;
+        }
+        const u32x4_t a0h = *reinterpret_cast<const u32x4_t*>(&snapslot->AQ[0][0][n][32 * j + 8 * g]);
+        const u32x4_t a0l = *reinterpret_cast<const u32x4_t*>(&snapslot->AQ[1][0][n][32 * j + 8 * g]);
+        const u32x4_t a1h = *reinterpret_cast<const u32x4_t*>(&snapslot->AQ[0][1][n][32 * j + 8 * g]);
+        const u32x4_t a1l = *reinterpret_cast<const u32x4_t*>(&snapslot->AQ[1][1][n][32 * j + 8 * g]);
+        W = mfma(a0h, gh, W); Y = mfma(a1h, gh, Y);
+        W = mfma(a0h, gl, W); Y = mfma(a1h, gl, Y);
+        W = mfma(a0l, gh, W); Y = mfma(a1l, gh, Y);
+      }
+    }
+  }
   // At, Qt, Mka, Mkr, v^T are dead now: fetch the next chunk's into the same registers
   if (next != nullptr) {
     next_ready();
@@ -417,42 +532,41 @@ __device__ __forceinline__ void consume(Consumer& C, Ops& o, const Slot* __restr
   Y = mfma(o.Br, sHH, Y);
   Y = mfma(o.Br, sL0, Y);                     // Y^T += Mbr^T SA^T
   if (next != nullptr) o.Br = *reinterpret_cast<const u32x4_t*>(&next->Mt[2][lane]);
-  // state snapshot for `length` (one chunk per sequence)
-  if (is_snap) {
-    const bool keep = slot->keep_snap != 0;
+  if constexpr (!REV) {
+    // state snapshot for `length` (one chunk per sequence)
+    if (is_snap) {
+      const bool keep = slot->keep_snap != 0;
 #pragma unroll
-    for (int tile = 0; tile < 4; ++tile) {
-      const u32x4_t sb = *reinterpret_cast<const u32x4_t*>(&snapslot->BT[0][tile][lane]);
-      const u32x4_t sk = *reinterpret_cast<const u32x4_t*>(&snapslot->BT[1][tile][lane]);
-      f32x4_t acc = keep ? C.S[tile] : zero4;
-      acc = mfma(sb, sHH, acc);
-      acc = mfma(sk, vv, acc);
-      acc = mfma(sb, sL0, acc);
-      const float4 sg = *reinterpret_cast<const float4*>(&snapslot->gamma[16 * tile + 4 * g]);
-      acc[0] *= sg.x; acc[1] *= sg.y; acc[2] *= sg.z; acc[3] *= sg.w;
-      const size_t off = (((size_t)b * A.H + h) * 64 + 16 * C.q + n) * 64 + 16 * tile + 4 * g;
-      if (A.st_f32) {
-        float4 ov = q2drop ? make_float4(0.f, 0.f, 0.f, 0.f) : make_float4(acc[0], acc[1], acc[2], acc[3]);
-        *reinterpret_cast<float4*>(reinterpret_cast<float*>(A.new_s) + off) = ov;
-      } else {
-        uint2 ov = q2drop ? make_uint2(0u, 0u) : make_uint2(pack_rn(acc[0], acc[1]), pack_rn(acc[2], acc[3]));
-        *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(A.new_s) + off) = ov;
+      for (int tile = 0; tile < 4; ++tile) {
+        const u32x4_t sb = *reinterpret_cast<const u32x4_t*>(&snapslot->BT[0][tile][lane]);
+        const u32x4_t sk = *reinterpret_cast<const u32x4_t*>(&snapslot->BT[1][tile][lane]);
+        f32x4_t acc = keep ? C.S[tile] : zero4;
+        acc = mfma(sb, sHH, acc);
+        acc = mfma(sk, vv, acc);
+        acc = mfma(sb, sL0, acc);
+        const float4 sg = *reinterpret_cast<const float4*>(&snapslot->gamma[16 * tile + 4 * g]);
+        acc[0] *= sg.x; acc[1] *= sg.y; acc[2] *= sg.z; acc[3] *= sg.w;
+        store_state_tile(A.new_s, A.st_f32, state_off(A, b, h, C.q, lane, tile), q2drop ? zero4 : acc);
       }
     }
-  }
-  // state update, tile by tile: rows = keys.  S <- (S + Bh^T SA^T + Kh^T V^T) . gamma
-  if (!keep_end) {
-    asm volatile("" ::: "memory");   // keep this a (rare, uniform) branch instead of 16 selects on the hot path
+    // a reset inside the chunk cuts the entering state off
+    if (!keep_end) {
+      asm volatile("" ::: "memory");   // keep this a (rare, uniform) branch instead of 16 selects on the hot path
 #pragma unroll
-    for (int tile = 0; tile < 4; ++tile) C.S[tile] = zero4;   // a reset inside the chunk cuts the entering state off
+      for (int tile = 0; tile < 4; ++tile) C.S[tile] = zero4;
+    }
   }
+  // state update, tile by tile: rows = keys.  forward S <- (S + Bh^T SA^T + Kh^T V^T) . gamma,
+  // reverse G <- Gh + At^T DSA^T + Qt^T DY^T
 #pragma unroll
   for (int tile = 0; tile < 4; ++tile) {
     f32x4_t acc = C.S[tile];
     acc = mfma(bt[0][tile], sHH, acc);
     acc = mfma(bt[1][tile], vv, acc);
     acc = mfma(bt[0][tile], sL0, acc);
-    acc[0] *= gm[tile].x; acc[1] *= gm[tile].y; acc[2] *= gm[tile].z; acc[3] *= gm[tile].w;
+    if constexpr (!REV) {
+      acc[0] *= gm[tile].x; acc[1] *= gm[tile].y; acc[2] *= gm[tile].z; acc[3] *= gm[tile].w;
+    }
     C.S[tile] = acc;
   }
   // outputs: register i is token 4g+i, lanes n = 16 consecutive values
@@ -478,47 +592,24 @@ __device__ __forceinline__ void consume(Consumer& C, Ops& o, const Slot* __restr
       }
     }
   }
-  oc.y += CK * oc.tok_bytes;
-  if (oc.sa != nullptr) oc.sa += 2 * CK * oc.tok_bytes;
-}
-
-__device__ __forceinline__ void load_state(Consumer& C, const Wkv7Args& A, int64_t b, int64_t h) {
-  const int n = C.lane & 15, g = C.lane >> 4;
-#pragma unroll
-  for (int tile = 0; tile < 4; ++tile) {
-    const size_t off = (((size_t)b * A.H + h) * 64 + 16 * C.q + n) * 64 + 16 * tile + 4 * g;
-    if (A.st_f32) {
-      const float4 x = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(A.s) + off);
-      C.S[tile][0] = x.x; C.S[tile][1] = x.y; C.S[tile][2] = x.z; C.S[tile][3] = x.w;
-    } else {
-      const uint2 x = *reinterpret_cast<const uint2*>(reinterpret_cast<const uint16_t*>(A.s) + off);
-      C.S[tile][0] = __uint_as_float(x.x << 16); C.S[tile][1] = __uint_as_float(x.x & 0xffff0000u);
-      C.S[tile][2] = __uint_as_float(x.y << 16); C.S[tile][3] = __uint_as_float(x.y & 0xffff0000u);
-    }
-  }
-}
-
-__device__ __forceinline__ void store_state0(const Consumer& C, const Wkv7Args& A, int64_t b, int64_t h, bool zero) {
-  // length == 0: the returned state is the input state (rwkv7.py:203), or the reset state under the associative rule
-  const int n = C.lane & 15, g = C.lane >> 4;
-#pragma unroll
-  for (int tile = 0; tile < 4; ++tile) {
-    const size_t off = (((size_t)b * A.H + h) * 64 + 16 * C.q + n) * 64 + 16 * tile + 4 * g;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const float x = zero ? 0.f : C.S[tile][i];
-      if (A.st_f32) reinterpret_cast<float*>(A.new_s)[off + i] = x;
-      else reinterpret_cast<uint16_t*>(A.new_s)[off + i] = f32_to_bf16(x);
-    }
+  if constexpr (!REV) {
+    oc.y += CK * oc.tok_bytes;
+    if (oc.sa != nullptr) oc.sa += 2 * CK * oc.tok_bytes;
+  } else {
+    oc.y -= CK * oc.tok_bytes;
+    oc.sa -= 2 * CK * oc.tok_bytes;
   }
 }
 
 }  // namespace
 
-// Slot c % RING holds chunk c.  Producer p fills it once every consumer has released chunk c - RING, then
-// publishes ready = c + 1; consumers take chunks in order.  Every wait is for a strictly earlier chunk, so the
-// hand-shake cannot cycle.
-__global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_fwd_kernel(Wkv7Args A) {
+// Chunks are handled in sequence order in the forward pass and from the last one down in the reverse sweep; step j
+// handles chunk c(j) in slot j % RING.  Producer p fills the slot once every consumer has released step j - RING,
+// then publishes ready = j + 1; consumers take the steps in order.  Every wait is for a strictly earlier step, so
+// the hand-shake cannot cycle.
+template <bool REV>
+__global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_kernel(Wkv7Args A) {
+  using SnapSlot = SnapSlotT<REV>;
   extern __shared__ __align__(16) unsigned char smem_raw[];
   Slot* slots = reinterpret_cast<Slot*>(smem_raw);
   SnapSlot* snapslot = reinterpret_cast<SnapSlot*>(smem_raw + RING * sizeof(Slot));
@@ -528,39 +619,72 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_fwd_kernel(Wk
   const int64_t b = blockIdx.x / A.H, h = blockIdx.x % A.H;
   int64_t L = A.length ? (int64_t)A.length[b] : A.T;
   L = L < A.T ? L : A.T;
-  const int64_t nchunks = (A.T + CK - 1) / CK;
+  const int nch = (int)((A.T + CK - 1) / CK);
+  // the returned state is the reset state there (associative-scan rule), a constant
+  const bool q2drop = (A.flags & 1u) && L < A.T && A.ns != nullptr && A.ns[b * A.T + L] != 0;
+  // reverse sweep: does a cotangent of the returned state enter at token length-1?
+  const bool inject = REV && A.gs_out != nullptr && !q2drop;
   if (threadIdx.x < sizeof(Sync) / sizeof(int)) reinterpret_cast<int*>(sy)[threadIdx.x] = 0;
   __syncthreads();
 
   if (wave < NCONS) {
     // the chunk-to-chunk dependency runs through the consumers: let them issue ahead of the producers
     __builtin_amdgcn_s_setprio(3);
-    const bool q2drop = (A.flags & 1u) && L < A.T && A.ns != nullptr && A.ns[b * A.T + L] != 0;
     Consumer C;
     C.q = wave;
     C.lane = lane;
-    load_state(C, A, b, h);
-    if (L == 0) store_state0(C, A, b, h, q2drop);
+    const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+    if constexpr (!REV) {
+#pragma unroll
+      for (int tile = 0; tile < 4; ++tile) C.S[tile] = load_state_tile(A.s, A.st_f32, state_off(A, b, h, wave, lane, tile));
+      // length == 0: the returned state is the input state (rwkv7.py:203), or the reset state under the associative rule
+      if (L == 0) {
+#pragma unroll
+        for (int tile = 0; tile < 4; ++tile)
+          store_state_tile(A.new_s, A.st_f32, state_off(A, b, h, wave, lane, tile), q2drop ? zero4 : C.S[tile]);
+      }
+    } else {
+#pragma unroll
+      for (int tile = 0; tile < 4; ++tile) C.S[tile] = zero4;
+    }
+    const int64_t first_tok = REV ? (int64_t)(nch - 1) * CK : 0;
     OutCursor oc;
     oc.tok_bytes = (size_t)A.H * 64 * 2;
-    oc.y = reinterpret_cast<char*>(A.out) + (((size_t)b * A.T) * A.H + h) * 64 * 2;
-    oc.sa = A.sa ? reinterpret_cast<char*>(A.sa) + (((size_t)b * A.T) * A.H + h) * 64 * 4 : nullptr;
+    const size_t el0 = (((size_t)b * A.T + first_tok) * A.H + h) * 64;
+    if constexpr (!REV) {
+      oc.y = reinterpret_cast<char*>(A.out) + el0 * 2;
+      oc.sa = A.sa ? reinterpret_cast<char*>(A.sa) + el0 * 4 : nullptr;
+    } else {
+      oc.y = reinterpret_cast<char*>(A.gv) + el0 * 2;
+      oc.sa = reinterpret_cast<char*>(A.dsa) + el0 * 4;
+    }
     oc.voff = (uint32_t)((4 * (lane >> 4)) * (int)A.H * 64 + 16 * wave + (lane & 15));
-    const int csnap = L >= 1 ? (int)((L - 1) / CK) : -1;
-    const int nch = (int)nchunks;
+    const int csnap = (L >= 1 && (!REV || inject)) ? (int)((L - 1) / CK) : -1;
     Ops ops;
     if (nch > 0) {
       wait_ready(sy, 0, 1);
       load_ops(ops, &slots[0], wave, lane);
     }
-    for (int c = 0; c < nch; ++c) {
+    for (int j = 0; j < nch; ++j) {
+      const int c = REV ? nch - 1 - j : j;
       const int nvalid = (c + 1 < nch || A.T % CK == 0) ? CK : (int)(A.T % CK);
-      const int si = c % RING, sn = (c + 1) % RING;
-      const Slot* next = (c + 1 < nch) ? &slots[sn] : nullptr;
-      consume(C, ops, &slots[si], next, snapslot, A, b, h, nvalid, c == csnap, q2drop, oc,
-              [&]() { wait_ready(sy, sn, c + 2); });
+      const int si = j % RING, sn = (j + 1) % RING;
+      const Slot* next = (j + 1 < nch) ? &slots[sn] : nullptr;
+      consume<REV>(C, ops, &slots[si], next, snapslot, A, b, h, nvalid, c == csnap, q2drop, oc,
+                   [&]() { wait_ready(sy, sn, j + 2); });
       // every LDS read of slot si has returned: its data went into the MFMAs above
-      if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], c + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+      if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+    if constexpr (REV) {
+      // cotangent of the input state; with length == 0 the returned state is the input state itself
+      const bool pass = L == 0 && inject;
+#pragma unroll
+      for (int tile = 0; tile < 4; ++tile) {
+        const size_t off = state_off(A, b, h, wave, lane, tile);
+        f32x4_t gsv = C.S[tile];
+        if (pass) gsv += load_state_tile(A.gs_out, A.st_f32, off);
+        store_state_tile(A.gs, A.st_f32, off, gsv);
+      }
     }
   } else {
     const int p = wave - NCONS;
@@ -568,28 +692,36 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_fwd_kernel(Wk
     P.lane = lane;
     make_sel(P.sel, lane);
     Raw raw;
-    if (p < nchunks) load_raw(raw, A, b, h, (int64_t)p * CK, lane);
-    for (int64_t c = p; c < nchunks; c += NPROD) {
-      const int64_t c0 = c * CK;
-      const ChunkFlags F = chunk_flags(A.ns, A.flags, A.T, b, c0, L, lane);
-      const int si = (int)(c % RING);
+    if (p < nch) load_raw<REV>(raw, A, b, h, (int64_t)(REV ? nch - 1 - p : p) * CK, lane);
+    for (int j = p; j < nch; j += NPROD) {
+      const int c = REV ? nch - 1 - j : j;
+      const int64_t c0 = (int64_t)c * CK;
+      ChunkFlags F = chunk_flags(A.ns, A.flags, A.T, b, c0, L, lane);
+      if (REV && !inject) F.snap = -1;
+      const int si = j % RING;
       Slot* slot = &slots[si];
-      if (c >= RING) wait_consumed(sy, si, (int)(c - RING) + 1, lane);
-      produce(P, raw, F, slot, snapslot);
-      if (c + NPROD < nchunks) load_raw(raw, A, b, h, c0 + NPROD * CK, lane);
+      if (j >= RING) wait_consumed(sy, si, j - RING + 1, lane);
+      produce<REV>(P, raw, F, slot, snapslot);
+      if (j + NPROD < nch) load_raw<REV>(raw, A, b, h, (int64_t)(REV ? c - NPROD : c + NPROD) * CK, lane);
       // the release orders this wave's LDS writes before the sequence number
-      if (lane == 0) __hip_atomic_store(&sy->ready[si], (int)c + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+      if (lane == 0) __hip_atomic_store(&sy->ready[si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
   }
 }
 
-hipError_t launch_wkv7_chunk_fwd(const Wkv7Args& A, hipStream_t stream) {
-  const size_t smem = RING * sizeof(Slot) + sizeof(SnapSlot) + sizeof(Sync);
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(wkv7_chunk_fwd_kernel),
+template <bool REV>
+static hipError_t launch_chunk(const Wkv7Args& A, hipStream_t stream) {
+  const size_t smem = RING * sizeof(Slot) + sizeof(SnapSlotT<REV>) + sizeof(Sync);
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(wkv7_chunk_kernel<REV>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
   if (e != hipSuccess) return e;
-  hipLaunchKernelGGL(wkv7_chunk_fwd_kernel, dim3((unsigned)(A.B * A.H)), dim3(64 * (NCONS + NPROD)), smem, stream, A);
+  hipLaunchKernelGGL(wkv7_chunk_kernel<REV>, dim3((unsigned)(A.B * A.H)), dim3(64 * (NCONS + NPROD)), smem, stream, A);
   return hipGetLastError();
 }
+
+hipError_t launch_wkv7_chunk_fwd(const Wkv7Args& A, hipStream_t stream) { return launch_chunk<false>(A, stream); }
+
+// Reverse sweep of the backward pass: gv, the workspace dsa (cotangent of sa per token) and gs.
+hipError_t launch_wkv7_chunk_bwd_a(const Wkv7Args& A, hipStream_t stream) { return launch_chunk<true>(A, stream); }
 
 }  // namespace hiprwkv

@@ -333,20 +333,28 @@ hipError_t launch_wkv7_seq_fwd(const Wkv7Args& A, hipStream_t stream) {
   return hipGetLastError();
 }
 
-hipError_t launch_wkv7_seq_bwd(const Wkv7Args& A, hipStream_t stream) {
-  constexpr size_t sa_ = seq_smem_bytes<6, 2, BWA_CH>();
-  constexpr size_t sb_ = seq_smem_bytes<9, 4, BWB_CH>();
-  constexpr size_t sc_ = seq_smem_bytes<12, 3, BWC_CH>();
-  hipError_t e;
-  if ((e = set_smem(reinterpret_cast<const void*>(wkv7_seq_bwd_a_kernel), sa_)) != hipSuccess) return e;
-  if ((e = set_smem(reinterpret_cast<const void*>(wkv7_seq_bwd_b_kernel), sb_)) != hipSuccess) return e;
-  if ((e = set_smem(reinterpret_cast<const void*>(wkv7_seq_bwd_c_kernel), sc_)) != hipSuccess) return e;
-  const dim3 grid((unsigned)(A.B * A.H)), block(SEQ_THREADS);
-  hipLaunchKernelGGL(wkv7_seq_bwd_a_kernel, grid, block, sa_, stream, A);
-  if ((e = hipGetLastError()) != hipSuccess) return e;
-  hipLaunchKernelGGL(wkv7_seq_bwd_b_kernel, grid, block, sb_, stream, A);
-  if ((e = hipGetLastError()) != hipSuccess) return e;
-  hipLaunchKernelGGL(wkv7_seq_bwd_c_kernel, grid, block, sc_, stream, A);
+// The three backward sweeps, in the order they must run (A, B, C).
+hipError_t launch_wkv7_seq_bwd_a(const Wkv7Args& A, hipStream_t stream) {
+  constexpr size_t smem = seq_smem_bytes<6, 2, BWA_CH>();
+  hipError_t e = set_smem(reinterpret_cast<const void*>(wkv7_seq_bwd_a_kernel), smem);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(wkv7_seq_bwd_a_kernel, dim3((unsigned)(A.B * A.H)), dim3(SEQ_THREADS), smem, stream, A);
+  return hipGetLastError();
+}
+
+hipError_t launch_wkv7_seq_bwd_b(const Wkv7Args& A, hipStream_t stream) {
+  constexpr size_t smem = seq_smem_bytes<9, 4, BWB_CH>();
+  hipError_t e = set_smem(reinterpret_cast<const void*>(wkv7_seq_bwd_b_kernel), smem);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(wkv7_seq_bwd_b_kernel, dim3((unsigned)(A.B * A.H)), dim3(SEQ_THREADS), smem, stream, A);
+  return hipGetLastError();
+}
+
+hipError_t launch_wkv7_seq_bwd_c(const Wkv7Args& A, hipStream_t stream) {
+  constexpr size_t smem = seq_smem_bytes<12, 3, BWC_CH>();
+  hipError_t e = set_smem(reinterpret_cast<const void*>(wkv7_seq_bwd_c_kernel), smem);
+  if (e != hipSuccess) return e;
+  hipLaunchKernelGGL(wkv7_seq_bwd_c_kernel, dim3((unsigned)(A.B * A.H)), dim3(SEQ_THREADS), smem, stream, A);
   return hipGetLastError();
 }
 

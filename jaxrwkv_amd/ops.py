@@ -71,8 +71,10 @@ def wkv7_fwd(r, w, k, v, a, b, s, length=None, new_starts=None, compat=True, wan
     return new_s, y, sa
 
 
-def wkv7_bwd(r, w, k, v, a, b, s, length, new_starts, gy, sa, gs_out=None, compat=True):
-    """Cotangents (gr, gw, gk, gv, ga, gb, gs) of ``wkv7_fwd`` for cotangents gy of y and gs_out of new_s."""
+def wkv7_bwd(r, w, k, v, a, b, s, length, new_starts, gy, sa, gs_out=None, compat=True, force_seq=False):
+    """Cotangents (gr, gw, gk, gv, ga, gb, gs) of ``wkv7_fwd`` for cotangents gy of y and gs_out of new_s.
+
+    bf16 inputs use the chunked MFMA kernels where they exist unless ``force_seq`` asks for the sequential ones."""
     lib = _lib.load()
     io = r.dtype
     r, w, k, v, a, b, gy = (_dev(x, io) for x in (r, w, k, v, a, b, gy))
@@ -87,7 +89,8 @@ def wkv7_bwd(r, w, k, v, a, b, s, length, new_starts, gy, sa, gs_out=None, compa
     ws = torch.empty(nbytes, dtype=torch.uint8, device=r.device)
     rc = lib.hiprwkv_wkv7_bwd(_stream(), _DT[io], _DT[s.dtype], B, T, H, N, _p(w), _p(r), _p(k), _p(v), _p(a), _p(b),
                               _p(s), _p(length), _p(new_starts), _p(gy), _p(sa), _p(gs_out),
-                              _p(gw), _p(gr), _p(gk), _p(gv), _p(ga), _p(gb), _p(gs), _p(ws), nbytes, _flags(compat))
+                              _p(gw), _p(gr), _p(gk), _p(gv), _p(ga), _p(gb), _p(gs), _p(ws), nbytes,
+                              _flags(compat, force_seq))
     _lib.check(rc, "hiprwkv_wkv7_bwd")
     return gr, gw, gk, gv, ga, gb, gs
 
