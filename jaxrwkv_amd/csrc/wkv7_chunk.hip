@@ -307,27 +307,32 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
   }
   // ---- triangular masks: forward keeps earlier rows m for column n, the reverse sweep later rows
   const int n = t;
-  {
-    const bool dropy = !REV && slow && F.compat && ((F.ns >> (n + 1)) & 1u);   // y[n] is defined as zero
+  auto mask_tiles = [&](int i, bool lt, bool le, bool gt, bool ge) {
+    Gab[i] = lt ? Gab[i] : 0.f;
+    GabT[i] = gt ? GabT[i] : 0.f;
+    if constexpr (!REV) {
+      G1[i] = lt ? G1[i] : 0.f;
+      G2[i] = le ? G2[i] : 0.f;
+      G3[i] = le ? G3[i] : 0.f;
+    } else {
+      G1[i] = ge ? G1[i] : 0.f;
+      G2[i] = gt ? G2[i] : 0.f;
+      G3[i] = ge ? G3[i] : 0.f;
+    }
+  };
+  if (!slow) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int m = 4 * g + i;
-      bool lt = m < n, le = m <= n, gt = m > n, ge = m >= n;
-      if (slow) {
-        const bool same = seg_of(F.ns, m) == seg_of(F.ns, n);
-        lt = lt && same; le = le && same; gt = gt && same; ge = ge && same;
-      }
-      Gab[i] = lt ? Gab[i] : 0.f;
-      GabT[i] = gt ? GabT[i] : 0.f;
-      if constexpr (!REV) {
-        G1[i] = lt ? G1[i] : 0.f;
-        G2[i] = (le && !dropy) ? G2[i] : 0.f;
-        G3[i] = (le && !dropy) ? G3[i] : 0.f;
-      } else {
-        G1[i] = ge ? G1[i] : 0.f;
-        G2[i] = gt ? G2[i] : 0.f;
-        G3[i] = ge ? G3[i] : 0.f;
-      }
+      mask_tiles(i, m < n, m <= n, m > n, m >= n);
+    }
+  } else {
+    const bool keepy = REV || !(F.compat && ((F.ns >> (n + 1)) & 1u));   // forward: y[n] may be defined as zero
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int m = 4 * g + i;
+      const bool same = seg_of(F.ns, m) == seg_of(F.ns, n);
+      mask_tiles(i, (m < n) && same, (m <= n) && same && keepy, (m > n) && same, (m >= n) && same);
     }
   }
   // ---- (I - M)^{-1} = (I + M^8)(I + M^4)(I + M^2)(I + M) in single bf16; forward M = Mba, reverse M = Mba^T
