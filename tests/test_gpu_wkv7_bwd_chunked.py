@@ -3,8 +3,10 @@ vector-Jacobian product on bf16-rounded inputs, and against the sequential fp32 
 
 Tolerances: cotangents are rounded to bf16 on output (one ulp = 2^-7 relative); the chunked sweeps feed fp32
 quantities to the matrix cores as bf16 hi+lo pairs (about 16 mantissa bits), so absolute errors are a few 1e-4 of
-the tensor's rms (1e-3 for the decay gradient, which comes out of a cancellation).  gs is fp32: rtol 1e-4,
-atol 1e-4 x rms.
+the tensor's rms.  The decay gradient is the exception: it is a running sum over the rest of the sequence of
+O(10) terms that now carry 2^-16 relative errors each, minus two such terms, so single elements are off by up to
+1e-2 of its rms (about one bf16 ulp of a typical element; rel-rms error 2e-3 against 1.7e-3 for the sequential
+fp32 sweeps, whose only error is the bf16 rounding of the output).  gs is fp32: rtol 1e-4, atol 1e-4 x rms.
 """
 import numpy as np
 import pytest
@@ -16,7 +18,7 @@ from tests.inputs import wkv7_inputs
 
 pytestmark = pytest.mark.gpu
 NAMES = ("r", "w", "k", "v", "a", "b", "s")
-ATOL = dict(r=5e-4, w=2e-3, k=5e-4, v=5e-4, a=5e-4, b=1e-3, s=1e-4)
+ATOL = dict(r=5e-4, w=1e-2, k=5e-4, v=5e-4, a=5e-4, b=1e-3, s=1e-4)
 RTOL = dict(r=2.0 ** -7, w=2.0 ** -7, k=2.0 ** -7, v=2.0 ** -7, a=2.0 ** -7, b=2.0 ** -7, s=1e-4)
 
 
