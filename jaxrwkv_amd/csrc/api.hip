@@ -104,12 +104,12 @@ int hiprwkv_wkv7_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64
   A.e2 = reinterpret_cast<float*>(ws + one);
   A.e3 = reinterpret_cast<float*>(ws + 2 * one);
   // Three sweeps: A (reverse) -> gv, dsa, gs; B (forward) -> gr, ga, e2, e3; C (reverse) -> gk, gb, gw.
-  // bf16 I/O runs sweeps A and B on the chunked MFMA kernels.
+  // bf16 I/O runs all three on the chunked MFMA kernels.
   const bool chunked = io_dtype == HIPRWKV_BF16 && !(flags & HIPRWKV_FORCE_SEQ);
   hipStream_t st = static_cast<hipStream_t>(stream);
   hipError_t e = chunked ? launch_wkv7_chunk_bwd_a(A, st) : launch_wkv7_seq_bwd_a(A, st);
   if (e == hipSuccess) e = chunked ? launch_wkv7_chunk_bwd_b(A, st) : launch_wkv7_seq_bwd_b(A, st);
-  if (e == hipSuccess) e = launch_wkv7_seq_bwd_c(A, st);
+  if (e == hipSuccess) e = chunked ? launch_wkv7_chunk_bwd_c(A, st) : launch_wkv7_seq_bwd_c(A, st);
   if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "wkv7_bwd: %s", hipGetErrorString(e));
   return HIPRWKV_OK;
 }
