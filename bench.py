@@ -141,7 +141,7 @@ def bench_wkv7(torch, ops, args):
             new_s, y, sa = ops.wkv7_fwd(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], x["length"],
                                         x["new_starts"], compat=True, want_sa=True, force_seq=args.seq)
             return ops.wkv7_bwd(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], x["length"], x["new_starts"],
-                                x["dy"], sa, None, compat=True)
+                                x["dy"], sa, None, compat=True, force_seq=args.seq)
         n2 = max(2, args.steps // 4)
         wall2, _ = time_region(torch, fwd_bwd, n2, 1)
         ms2 = 1e3 * wall2 / n2
@@ -149,7 +149,9 @@ def bench_wkv7(torch, ops, args):
         fb_bytes = 20 * tokens * H * N * 2 + 4 * B * H * N * N * 4
         out["fwd_bwd"] = {"tokens_per_s": tokens / (ms2 * 1e-3), "ms_per_step": ms2,
                           "hbm_frac": fb_bytes / (ms2 * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": fb_bytes,
-                          "note": "backward = three sequential fp32 sweeps (no chunked MFMA backward yet)"}
+                          "note": "backward = three sweeps (reverse, forward, reverse), " +
+                                  ("sequential fp32 VALU kernels" if args.seq else "chunked MFMA kernels") +
+                                  "; dsa, e2, e3 pass through an fp32 workspace"}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
         out["cpu_baseline_sequential"] = cpu_baseline_sequential()
@@ -174,7 +176,8 @@ def bench_wkv6(torch, ops, args):
     fwd_bytes = 5 * tokens * H * N * 2 + 2 * b6 * H * N * N * 4 + b6 * t6
     out = base_record("WKV6 fwd tokens/s (B16 T2048 H32 N64 bf16)", tokens / (ms_step * 1e-3), ms_step, args, "bf16",
                       "isolated WKV6 op, B=16 T=2048 H=32 N=64 bf16, zero state, new_starts~Bernoulli(1/512) "
-                      "(BASELINE configs[2])", {"kernel": "sequential fp32 VALU"})
+                      "(BASELINE configs[2])",
+                      {"kernel": "chunked MFMA forward (bf16 hi+lo operands, fp32 accumulate); sequential fp32 backward"})
     out["roofline"] = roofline(fwd_bytes, kern_ms, None)
     if not args.no_bwd:
         fb = lambda: ops.wkv6_bwd(r, k, v, w, u, s, None, ns, dy, None, compat=True)
