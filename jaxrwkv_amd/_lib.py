@@ -11,6 +11,7 @@ LIB_PATH = os.path.join(HERE, "libhiprwkv.so")
 F32, BF16 = 0, 1
 COMPAT_ASSOC = 1
 FORCE_SEQ = 2
+NO_SMALL_T = 4
 
 _vp, _i64, _int, _u32, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_uint, ctypes.c_size_t
 

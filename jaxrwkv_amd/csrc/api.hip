@@ -62,10 +62,12 @@ int hiprwkv_wkv7_fwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64
   A.out = out; A.sa = sa; A.new_s = new_s;
   A.io_f32 = io_dtype == HIPRWKV_F32; A.st_f32 = state_dtype == HIPRWKV_F32;
   A.flags = flags;
-  // bf16 I/O runs on the chunked MFMA kernel; fp32 I/O (and HIPRWKV_FORCE_SEQ) on the exact sequential one
+  // T <= 8 (decode) runs on the small-T kernel; otherwise bf16 I/O on the chunked MFMA kernel and fp32 I/O (and
+  // HIPRWKV_FORCE_SEQ) on the exact sequential one
+  const bool small_t = T <= HIPRWKV_SMALL_T && !(flags & HIPRWKV_NO_SMALL_T);
   const bool chunked = io_dtype == HIPRWKV_BF16 && !(flags & HIPRWKV_FORCE_SEQ);
-  hipError_t e = chunked ? launch_wkv7_chunk_fwd(A, static_cast<hipStream_t>(stream))
-                         : launch_wkv7_seq_fwd(A, static_cast<hipStream_t>(stream));
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipError_t e = small_t ? launch_wkv7_small_t_fwd(A, st) : chunked ? launch_wkv7_chunk_fwd(A, st) : launch_wkv7_seq_fwd(A, st);
   if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "wkv7_fwd: %s", hipGetErrorString(e));
   return HIPRWKV_OK;
 }

@@ -45,16 +45,18 @@ def _length_ns(length, new_starts, B, T, device):
     return length, new_starts
 
 
-def _flags(compat, force_seq=False):
-    return (_lib.COMPAT_ASSOC if compat else 0) | (_lib.FORCE_SEQ if force_seq else 0)
+def _flags(compat, force_seq=False, small_t=True):
+    return ((_lib.COMPAT_ASSOC if compat else 0) | (_lib.FORCE_SEQ if force_seq else 0)
+            | (0 if small_t else _lib.NO_SMALL_T))
 
 
 # ----------------------------------------------------------------------------- WKV7
-def wkv7_fwd(r, w, k, v, a, b, s, length=None, new_starts=None, compat=True, want_sa=False, force_seq=False):
+def wkv7_fwd(r, w, k, v, a, b, s, length=None, new_starts=None, compat=True, want_sa=False, force_seq=False,
+             small_t=True):
     """r,w,k,v,a,b (B,T,H,N) fp32|bf16; s (B,H,N,N) fp32|bf16.  Returns (new_s, y, sa|None).
 
-    bf16 I/O runs on the chunked MFMA kernel, fp32 I/O on the sequential fp32 kernel; ``force_seq`` selects the
-    sequential kernel for bf16 I/O as well."""
+    T <= 8 runs on the small-T (decode) kernel unless ``small_t=False``; otherwise bf16 I/O runs on the chunked MFMA
+    kernel and fp32 I/O on the sequential fp32 kernel; ``force_seq`` selects the sequential kernel for bf16 I/O."""
     lib = _lib.load()
     io = r.dtype
     r, w, k, v, a, b = (_dev(x, io) for x in (r, w, k, v, a, b))
@@ -66,7 +68,8 @@ def wkv7_fwd(r, w, k, v, a, b, s, length=None, new_starts=None, compat=True, wan
     new_s = torch.empty_like(s)
     sa = torch.empty((B, T, H, N), dtype=torch.float32, device=r.device) if want_sa else None
     rc = lib.hiprwkv_wkv7_fwd(_stream(), _DT[io], _DT[s.dtype], B, T, H, N, _p(w), _p(r), _p(k), _p(v), _p(a), _p(b),
-                              _p(s), _p(length), _p(new_starts), _p(y), _p(sa), _p(new_s), _flags(compat, force_seq))
+                              _p(s), _p(length), _p(new_starts), _p(y), _p(sa), _p(new_s),
+                              _flags(compat, force_seq, small_t))
     _lib.check(rc, "hiprwkv_wkv7_fwd")
     return new_s, y, sa
 

@@ -20,7 +20,7 @@ def run_fwd(x, dtype, compat, state_dtype=torch.float32):
     from jaxrwkv_amd import ops
     t = {n: dev(x[n], dtype) for n in ("r", "w", "k", "v", "a", "b")}
     new_s, y, sa = ops.wkv7_fwd(t["r"], t["w"], t["k"], t["v"], t["a"], t["b"], dev(x["s"], state_dtype),
-                                dev(x["length"]), dev(x["new_starts"]), compat=compat, want_sa=True)
+                                dev(x["length"]), dev(x["new_starts"]), compat=compat, want_sa=True, small_t=False)
     torch.cuda.synchronize()
     return host(new_s), host(y), host(sa)
 

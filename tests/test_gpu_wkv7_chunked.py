@@ -24,7 +24,7 @@ def run(x, compat, state_dtype=torch.float32, force_seq=False, want_sa=True):
     t = {n: dev(x[n], torch.bfloat16) for n in ("r", "w", "k", "v", "a", "b")}
     new_s, y, sa = ops.wkv7_fwd(t["r"], t["w"], t["k"], t["v"], t["a"], t["b"], dev(x["s"], state_dtype),
                                 dev(x["length"]), dev(x["new_starts"]), compat=compat, want_sa=want_sa,
-                                force_seq=force_seq)
+                                force_seq=force_seq, small_t=False)
     torch.cuda.synchronize()
     return host(new_s), host(y), (host(sa) if sa is not None else None)
 
