@@ -7,7 +7,9 @@ tokens/s beside it, the HBM roofline of the dominant kernel and a bounded CPU ba
 associative-scan restatement on the host cores).
 
 `--workload wkv6` / `--workload wkv4` time the two secondary ops (B=16 T=2048 H=32 N=64 bf16, and B=32 T=4096
-C=2560 fp32) with the same JSON layout; the default, and the line the headline metric is quoted on, is wkv7.
+C=2560 fp32) with the same JSON layout; `--workload model7` runs the RWKV-7 1.5B-shaped full model through the torch
+harness (prefill B=16 T=4096, decode B=256 single-token steps, eager and from a captured HIP graph).  The default,
+and the line the headline metric is quoted on, is wkv7.
 """
 import argparse
 import json
@@ -213,12 +215,89 @@ def bench_wkv4(torch, ops, args):
     return out
 
 
+def bench_model7(torch, ops, args):
+    """BASELINE configs[4]: RWKV-7 1.5B-shaped random-init model through the torch harness with HipRWKV.inner_loop:
+    prefill B=16 T=4096 (new_starts ~ Bernoulli(1/2048)) and decode B=256 single-token steps from a carried state."""
+    from jaxrwkv_amd.model7 import RWKV7, randomize_weights
+    L, C, vocab = 24, 2048, 65536
+    bp, tp, bd = 16, 4096, 256
+    params = randomize_weights(0, L, C, vocab, dtype=torch.bfloat16, device="cuda", zero_init=True)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(0)
+    tokens = torch.randint(0, vocab, (bp, tp), device="cuda", generator=g)
+    ns = torch.rand((bp, tp), device="cuda", generator=g) < 1.0 / 2048
+    state = RWKV7.default_state(params, bp)
+    steps = max(1, args.steps // 10)
+
+    def prefill():
+        with torch.no_grad():
+            return RWKV7.forward(params, tokens, state, None, ns)
+
+    wall, _ = time_region(torch, prefill, steps, 1)
+    ms_p = 1e3 * wall / steps
+    # the recurrence alone at the same shape, all layers
+    x = {n: torch.randn((bp, tp, C // N, N), device="cuda", generator=g).bfloat16() for n in ("r", "w", "k", "v", "a", "b")}
+    s0 = torch.zeros((bp, C // N, N, N), dtype=torch.bfloat16, device="cuda")
+    op = lambda: ops.wkv7_fwd(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], s0, None, ns, compat=True)
+    _, op_ms = time_region(torch, op, 5, 1)
+    del x
+    # decode
+    dtok = torch.randint(0, vocab, (bd, 1), device="cuda", generator=g)
+    dstate = (0.1 * torch.randn((bd, L, 2 + N, C), device="cuda", generator=g)).bfloat16()
+
+    def decode():
+        with torch.no_grad():
+            return RWKV7.forward(params, dtok, dstate, None, None)
+
+    dsteps = max(4, args.steps)
+    wall_d, _ = time_region(torch, decode, dsteps, 2)
+    ms_d = 1e3 * wall_d / dsteps
+    xd = {n: torch.randn((bd, 1, C // N, N), device="cuda", generator=g).bfloat16() for n in ("r", "w", "k", "v", "a", "b")}
+    sd = torch.zeros((bd, C // N, N, N), dtype=torch.bfloat16, device="cuda")
+    opd = lambda: ops.wkv7_fwd(xd["r"], xd["w"], xd["k"], xd["v"], xd["a"], xd["b"], sd, None, None, compat=True)
+    _, opd_ms = time_region(torch, opd, 20, 3)
+    # the same decode step replayed from a captured HIP graph (removes the host's launch overhead)
+    graph_ms = None
+    try:
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                decode()
+        torch.cuda.current_stream().wait_stream(side)
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            g_logits, g_state = decode()
+        torch.cuda.synchronize()
+        wall_g, _ = time_region(torch, gr.replay, dsteps, 2)
+        graph_ms = 1e3 * wall_g / dsteps
+        e_logits, e_state = decode()
+        torch.cuda.synchronize()
+        graph_ok = bool(torch.equal(g_logits, e_logits) and torch.equal(g_state, e_state))
+    except Exception as exc:      # graph capture is an optimisation of the harness, not of the op
+        graph_ok = f"capture failed: {type(exc).__name__}: {exc}"[:200]
+    out = base_record("RWKV7 1.5B-shaped prefill tokens/s (B16 T4096 bf16, HipRWKV)", bp * tp / (ms_p * 1e-3), ms_p,
+                      args, "bf16", "full model L=24 C=2048 H=32 N=64 vocab=65536, bf16 random-init weights, torch "
+                      "harness + HipRWKV.inner_loop; prefill B=16 T=4096 new_starts~Bernoulli(1/2048) (BASELINE configs[4])")
+    out["steps"], out["warmup"] = steps, 1
+    out["prefill"] = {"ms_per_step": ms_p, "wkv_ms_all_layers": L * op_ms, "wkv_fraction": L * op_ms / ms_p}
+    out["decode"] = {"tokens_per_s": bd / (ms_d * 1e-3), "ms_per_step": ms_d, "batch": bd,
+                     "wkv_ms_all_layers": L * opd_ms, "wkv_fraction": L * opd_ms / ms_d,
+                     "hip_graph_ms_per_step": graph_ms,
+                     "hip_graph_tokens_per_s": (bd / (graph_ms * 1e-3)) if graph_ms else None,
+                     "hip_graph_replay_equals_eager": graph_ok}
+    # roofline of the dominant hand-written kernel of this workload: the WKV7 forward at the prefill shape
+    tok_heads = bp * tp * (C // N)
+    out["roofline"] = roofline(7 * tok_heads * N * 2 + 2 * bp * (C // N) * N * N * 2 + bp * tp, op_ms, None)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", choices=("wkv7", "wkv6", "wkv4"), default="wkv7")
+    ap.add_argument("--workload", choices=("wkv7", "wkv6", "wkv4", "model7"), default="wkv7")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-bwd", action="store_true")
     ap.add_argument("--seq", action="store_true", help="WKV7: force the sequential fp32 VALU kernel")
@@ -242,7 +321,7 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    out = {"wkv7": bench_wkv7, "wkv6": bench_wkv6, "wkv4": bench_wkv4}[args.workload](torch, ops, args)
+    out = {"wkv7": bench_wkv7, "wkv6": bench_wkv6, "wkv4": bench_wkv4, "model7": bench_model7}[args.workload](torch, ops, args)
     print(json.dumps(out))
 
 

@@ -71,3 +71,36 @@ def test_rwkv7_0p1b_shape_fp32():
     assert rel_rms(st, rst) < 1e-3, rel_rms(st, rst)
     tvd = 0.5 * np.abs(softmax(lg) - softmax(rlg)).sum(-1)
     assert tvd.max() < 1e-3, tvd.max()
+
+
+def test_decode_step_in_a_hip_graph_replays_like_eager():
+    """A captured decode step (B=8, T=1) replayed several times with new tokens and the carried state, with eager work
+    and synchronisations between the replays, equals the eager step every time."""
+    from jaxrwkv_amd.model7 import RWKV7, randomize_weights
+    params = randomize_weights(11, 2, 128, 211, dtype=torch.bfloat16, device="cuda", zero_init=False)
+    B = 8
+    gen = torch.Generator("cuda").manual_seed(3)
+    tok = torch.randint(0, 211, (B, 1), device="cuda", generator=gen)
+    state = (0.1 * torch.randn((B, 2, 66, 128), device="cuda", generator=gen)).bfloat16()
+
+    def step():
+        with torch.no_grad():
+            return RWKV7.forward(params, tok, state, None, None)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        step()
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        g_logits, g_state = step()
+    for it in range(4):
+        tok.copy_(torch.randint(0, 211, (B, 1), device="cuda", generator=gen))
+        e_logits, e_state = step()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(g_logits, e_logits), it
+        assert torch.equal(g_state, e_state), it
+        state.copy_(e_state)                          # carry the state into the next step
