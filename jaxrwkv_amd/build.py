@@ -32,6 +32,23 @@ def build(verbose=True):
     return LIB
 
 
+def build_xla_ffi(verbose=True):
+    """Compile csrc/xla_ffi.cc (the XLA custom-call handlers) into libhiprwkv_xla.so next to libhiprwkv.so.
+    Needs the XLA FFI headers that ship with jax (``jax.ffi.include_dir()``); raises where jax is not installed."""
+    import jax  # noqa: F401  (only here: the rest of the package does not depend on jax)
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    out = os.path.join(HERE, "libhiprwkv_xla.so")
+    cmd = [hipcc, "-O2", "-std=c++17", "-fPIC", "-shared", "-x", "hip", "--offload-arch=gfx950",
+           "-I" + jax.ffi.include_dir(), os.path.join(CSRC, "xla_ffi.cc"), "-L" + HERE, "-l:libhiprwkv.so",
+           "-Wl,-rpath,$ORIGIN", "-o", out]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    return out
+
+
 if __name__ == "__main__":
     build()
+    if "--xla-ffi" in sys.argv[1:]:
+        build_xla_ffi()
     sys.exit(0)

@@ -64,3 +64,18 @@ def test_product_does_not_import_the_oracle():
             if f.endswith((".py", ".hip", ".h", ".cpp")):
                 src = open(os.path.join(dirpath, f)).read()
                 assert "oracle" not in src, f"{f} mentions the oracle"
+
+
+def test_xla_ffi_sources_agree_on_symbols_and_abi():
+    """The XLA handler translation unit cannot be compiled here (no XLA headers): check statically that the Python
+    binding registers exactly the handler symbols it defines and that it only calls functions the C ABI declares."""
+    import re
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    cc = open(os.path.join(root, "jaxrwkv_amd", "csrc", "xla_ffi.cc")).read()
+    py = open(os.path.join(root, "jaxrwkv_amd", "jax_ffi.py")).read()
+    header = open(os.path.join(root, "include", "hiprwkv.h")).read()
+    defined = set(re.findall(r"XLA_FFI_DEFINE_HANDLER_SYMBOL\((\w+),", cc))
+    registered = set(re.findall(r'"hip-wkv\d-(?:fwd|bwd)": "(\w+)"', py))
+    assert defined == registered and len(defined) == 6
+    for fn in set(re.findall(r"\b(hiprwkv_\w+)\(", cc)):
+        assert re.search(r"\b%s\(" % fn, header), fn
