@@ -172,7 +172,16 @@ int hiprwkv_wkv6_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64
   char* ws = static_cast<char*>(workspace);
   A.er = reinterpret_cast<float*>(ws);
   A.eI = reinterpret_cast<float*>(ws + align256((size_t)B * T * H * N * sizeof(float)));
-  hipError_t e = launch_wkv6_seq_bwd(A, static_cast<hipStream_t>(stream));
+  // Two sweeps: F (forward) -> gr, gu, er, eI; R (reverse) -> gk, gv, gw, gs.  bf16 I/O runs them on the chunked
+  // MFMA kernels.
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipError_t e;
+  if (io_dtype == HIPRWKV_BF16 && !(flags & HIPRWKV_FORCE_SEQ)) {
+    e = launch_wkv6_chunk_bwd_f(A, st);
+    if (e == hipSuccess) e = launch_wkv6_chunk_bwd_r(A, st);
+  } else {
+    e = launch_wkv6_seq_bwd(A, st);
+  }
   if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "wkv6_bwd: %s", hipGetErrorString(e));
   return HIPRWKV_OK;
 }

@@ -147,8 +147,10 @@ def wkv6_fwd(r, k, v, w, u, s, length=None, new_starts=None, compat=True, force_
     return new_s, y
 
 
-def wkv6_bwd(r, k, v, w, u, s, length, new_starts, gy, gs_out=None, compat=True):
-    """Cotangents (gr, gk, gv, gw, gu, gs) of ``wkv6_fwd``; gu is summed over the batch here."""
+def wkv6_bwd(r, k, v, w, u, s, length, new_starts, gy, gs_out=None, compat=True, force_seq=False):
+    """Cotangents (gr, gk, gv, gw, gu, gs) of ``wkv6_fwd``; gu is summed over the batch here.
+
+    bf16 inputs run on the chunked MFMA kernels unless ``force_seq`` asks for the sequential fp32 ones."""
     lib = _lib.load()
     io = r.dtype
     B, T, H, N = r.shape
@@ -165,7 +167,7 @@ def wkv6_bwd(r, k, v, w, u, s, length, new_starts, gy, gs_out=None, compat=True)
     ws = torch.empty(nbytes, dtype=torch.uint8, device=r.device)
     rc = lib.hiprwkv_wkv6_bwd(_stream(), _DT[io], _DT[s.dtype], B, T, H, N, _p(r), _p(k), _p(v), _p(w), _p(u), _p(s),
                               _p(length), _p(new_starts), _p(gy), _p(gs_out), _p(gr), _p(gk), _p(gv), _p(gw), _p(gu),
-                              _p(gs), _p(ws), nbytes, _flags(compat))
+                              _p(gs), _p(ws), nbytes, _flags(compat, force_seq))
     _lib.check(rc, "hiprwkv_wkv6_bwd")
     return gr, gk, gv, gw, gu.sum(0).to(io), gs
 
