@@ -179,7 +179,7 @@ def bench_wkv6(torch, ops, args):
     out = base_record("WKV6 fwd tokens/s (B16 T2048 H32 N64 bf16)", tokens / (ms_step * 1e-3), ms_step, args, "bf16",
                       "isolated WKV6 op, B=16 T=2048 H=32 N=64 bf16, zero state, new_starts~Bernoulli(1/512) "
                       "(BASELINE configs[2])",
-                      {"kernel": "chunked MFMA forward (bf16 hi+lo operands, fp32 accumulate); sequential fp32 backward"})
+                      {"kernel": "chunked MFMA forward and backward (bf16 hi+lo operands, fp32 accumulate)"})
     out["roofline"] = roofline(fwd_bytes, kern_ms, None)
     if not args.no_bwd:
         fb = lambda: ops.wkv6_bwd(r, k, v, w, u, s, None, ns, dy, None, compat=True)
