@@ -70,6 +70,10 @@ __device__ __forceinline__ void split2(float x0, float x1, uint32_t& hi, uint32_
   lo = pack_rn(l0, l1);
 }
 
+// First statement of a rarely taken, wave-uniform branch (resets inside a chunk, the partial last chunk, the chunk
+// of token length-1): keeps the compiler from turning the branch into selects that every chunk would execute.
+__device__ __forceinline__ void rare_path() { asm volatile("" ::: "memory"); }
+
 template <int CTRL>
 __device__ __forceinline__ float dpp0(float x) {  // lanes without a source read 0
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true));

@@ -94,20 +94,26 @@ struct Raw {
   uint4 r[2], w[2], k[2], v[2], a[2], b[2];   // v holds dy in the reverse sweep
 };
 
+// Loads always touch a valid token (the last one of the sequence for lanes beyond it); mask_raw zeroes those lanes.
 template <bool REV>
 __device__ __forceinline__ void load_raw(Raw& x, const Wkv7Args& A, int64_t b, int64_t h, int64_t c0, int lane) {
   const int t = lane & 15, g = lane >> 4;
-  const uint4 z = make_uint4(0, 0, 0, 0);
-  if (c0 + t < A.T) {
-    const size_t off = ((((size_t)b * A.T + c0 + t) * A.H + h) * 64 + 8 * g) * 2;  // bytes
-    auto ld = [&](const void* p, uint4 (&o)[2]) {
-      o[0] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(p) + off);
-      o[1] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(p) + off + 64);
-    };
-    ld(A.r, x.r); ld(A.w, x.w); ld(A.k, x.k); ld(REV ? A.gy : A.v, x.v); ld(A.a, x.a); ld(A.b, x.b);
-  } else {
-    x.r[0] = x.r[1] = x.w[0] = x.w[1] = x.k[0] = x.k[1] = z;
-    x.v[0] = x.v[1] = x.a[0] = x.a[1] = x.b[0] = x.b[1] = z;
+  const int64_t tok = (c0 + t < A.T) ? c0 + t : A.T - 1;
+  const size_t off = ((((size_t)b * A.T + tok) * A.H + h) * 64 + 8 * g) * 2;  // bytes
+  auto ld = [&](const void* p, uint4 (&o)[2]) {
+    o[0] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(p) + off);
+    o[1] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(p) + off + 64);
+  };
+  ld(A.r, x.r); ld(A.w, x.w); ld(A.k, x.k); ld(REV ? A.gy : A.v, x.v); ld(A.a, x.a); ld(A.b, x.b);
+}
+__device__ __forceinline__ void mask_raw(Raw& x, int nvalid, int lane) {
+  if (nvalid != CK) {
+    rare_path();
+    if ((lane & 15) >= nvalid) {
+      const uint4 z = make_uint4(0, 0, 0, 0);
+      x.r[0] = x.r[1] = x.w[0] = x.w[1] = x.k[0] = x.k[1] = z;
+      x.v[0] = x.v[1] = x.a[0] = x.a[1] = x.b[0] = x.b[1] = z;
+    }
   }
 }
 
@@ -133,6 +139,7 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
   uint32_t keep_upd = 0xffffu, keep_snap = 0;
   if (F.snap >= 0) keep_snap = (2u << F.snap) - 1u;
   if (slow) {
+    rare_path();
     lastseg = seg_of(F.ns, 15);
     const int myseg = seg_of(F.ns, t);
     if (!REV) {
@@ -171,7 +178,10 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
     // ---- v^T (dy^T) of value tiles 2hf, 2hf+1: D[token][value] = sum_k V[token][k] sel[k][value]
     {
       uint4 vr = x.v[hf];
-      if (REV && drop_dy) vr = make_uint4(0, 0, 0, 0);
+      if (REV && slow) {
+        rare_path();
+        if (drop_dy) vr = make_uint4(0, 0, 0, 0);
+      }
       const u32x4_t vop = {vr.x, vr.y, vr.z, vr.w};
 #pragma unroll
       for (int x2 = 0; x2 < 2; ++x2) slot->VT[2 * hf + x2][lane] = plain_pack(mfma(vop, P.sel[x2], zero4));
@@ -182,14 +192,18 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
       float fw[8];
       unpack8(x.w[hf], fw);
 #pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        float l2 = fmaxf(-exp2_fast(fw[e] * LOG2E) * LOG2E, MIN_STEP_L2);
-        if (F.nvalid != CK) l2 = valid ? l2 : 0.f;
-        E[e] = row_scan(l2);
+      for (int e = 0; e < 8; ++e) fw[e] = fmaxf(-exp2_fast(fw[e] * LOG2E) * LOG2E, MIN_STEP_L2);
+      if (F.nvalid != CK) {
+        rare_path();
+#pragma unroll
+        for (int e = 0; e < 8; ++e) fw[e] = valid ? fw[e] : 0.f;
       }
+#pragma unroll
+      for (int e = 0; e < 8; ++e) E[e] = row_scan(fw[e]);
     }
     unpack8(x.a[hf], fa);
     if (slow) {
+      rare_path();
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const float base = __shfl(E[e], seg_src, 64);   // restart the cumulative decay at the last reset
@@ -227,7 +241,7 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
       *reinterpret_cast<float4*>(gp) = make_float4(E[0], E[1], E[2], E[3]);
       *reinterpret_cast<float4*>(gp + 4) = make_float4(E[4], E[5], E[6], E[7]);
     }
-    if (t == F.snap) {
+    if (F.snap >= 0 && t == F.snap) {
       float* gp = &snap->gamma[8 * g + 32 * hf];
       *reinterpret_cast<float4*>(gp) = make_float4(E[0], E[1], E[2], E[3]);
       *reinterpret_cast<float4*>(gp + 4) = make_float4(E[4], E[5], E[6], E[7]);
@@ -247,11 +261,13 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
         put(slot->AQ[0][0][t], r0h, true); put(slot->AQ[1][0][t], r0l, true);
         put(slot->AQ[0][1][t], r1h, true); put(slot->AQ[1][1][t], r1l, true);
       } else {
+        rare_path();
         put(slot->AQ[0][0][t], r0h, row0_keep); put(slot->AQ[1][0][t], r0l, row0_keep);
         put(slot->AQ[0][1][t], r1h, row1_keep); put(slot->AQ[1][1][t], r1l, row1_keep);
       }
       if constexpr (REV) {
         if (F.snap >= 0) {
+          rare_path();
           const bool sk = (keep_snap >> t) & 1u;
           put(snap->AQ[0][0][t], r0h, sk); put(snap->AQ[1][0][t], r0l, sk);
           put(snap->AQ[0][1][t], r1h, sk); put(snap->AQ[1][1][t], r1l, sk);
@@ -274,11 +290,13 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
           slot->BT[0][tile][lane] = join(plain_pack(d0h), plain_pack(d0l));
           slot->BT[1][tile][lane] = join(plain_pack(d1h), plain_pack(d1l));
         } else {
+          rare_path();
           slot->BT[0][tile][lane] = join(masked_pack(d0h, keep_upd), masked_pack(d0l, keep_upd));
           slot->BT[1][tile][lane] = join(masked_pack(d1h, keep_upd), masked_pack(d1l, keep_upd));
         }
         if constexpr (!REV) {
           if (F.snap >= 0) {
+            rare_path();
             snap->BT[0][tile][lane] = join(masked_pack(d0h, keep_snap), masked_pack(d0l, keep_snap));
             snap->BT[1][tile][lane] = join(masked_pack(d1h, keep_snap), masked_pack(d1l, keep_snap));
           }
@@ -327,6 +345,7 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
       mask_tiles(i, m < n, m <= n, m > n, m >= n);
     }
   } else {
+    rare_path();
     const bool keepy = REV || !(F.compat && ((F.ns >> (n + 1)) & 1u));   // forward: y[n] may be defined as zero
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -706,6 +725,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_kernel(Wkv7Ar
       const int si = j % RING;
       Slot* slot = &slots[si];
       if (j >= RING) wait_consumed(sy, si, j - RING + 1, lane);
+      mask_raw(raw, F.nvalid, lane);
       produce<REV>(P, raw, F, slot, snapslot);
       if (j + NPROD < nch) load_raw<REV>(raw, A, b, h, (int64_t)(REV ? c - NPROD : c + NPROD) * CK, lane);
       // the release orders this wave's LDS writes before the sequence number
