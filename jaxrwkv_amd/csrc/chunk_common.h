@@ -18,7 +18,7 @@ constexpr int NCONS = 4;          // consumer waves, one per 16 value rows
 constexpr int SPIN_LIMIT = 1 << 16;   // polls before a waiter gives up (milliseconds; a healthy wait is microseconds)
 constexpr float LOG2E = 1.44269504088896340736f;
 constexpr float MIN_STEP_L2 = -1.0e4f;          // keeps the running sum finite
-constexpr float MIN_CUM_L2 = -80.0f * LOG2E;    // 2^MIN_CUM_L2 = e^-80
+constexpr float MIN_CUM_L2 = -80.0f * LOG2E;    // floor of a chunk's total log2 decay: 2^MIN_CUM_L2 = e^-80
 
 // Hand-shake words.  ready[s] = c + 1 once chunk c is complete in slot s; consumed[q][s] = c + 1 once consumer
 // q no longer reads chunk c in slot s.  Waiting is a bounded poll, so that a broken hand-shake ends the kernel
@@ -88,6 +88,24 @@ __device__ __forceinline__ float row_scan(float x) {
   x += dpp0<0x118>(x);
   return x;
 }
+// E: inclusive running sums (log2 decay, <= 0, non-increasing along the row) of 8 channels over the 16 token lanes.
+// A channel whose total over the chunk is below MIN_CUM_L2 has all its steps of this chunk scaled by the same
+// factor so that the total becomes MIN_CUM_L2: 1/E stays finite in fp32 and the relative weights inside the chunk
+// keep their order, at the price of an inexact (weaker) decay for that channel in that chunk.
+__device__ __forceinline__ void cap_chunk_decay(float (&E)[8], int lane) {
+  bool over = false;
+#pragma unroll
+  for (int e = 0; e < 8; ++e) over = over || (E[e] < MIN_CUM_L2);
+  if (__ballot(over) != 0ull) {
+    rare_path();
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float tot = __shfl(E[e], (lane & 48) | 15, 64);
+      if (tot < MIN_CUM_L2) E[e] *= MIN_CUM_L2 / tot;
+    }
+  }
+}
+
 // value of the previous lane of the row; `first` in lane 0 of the row
 __device__ __forceinline__ float row_prev(float x, float first) {
   return __int_as_float(__builtin_amdgcn_update_dpp(__float_as_int(first), __float_as_int(x), 0x111, 0xf, 0xf, false));

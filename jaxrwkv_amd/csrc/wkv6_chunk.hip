@@ -18,9 +18,10 @@
 // new_starts inside a chunk restart the cumulative decay and mask the Gram tile (rare, uniform branch); `length`
 // snapshots use a second, masked set of update operands for the one chunk that holds token length-1.
 //
-// Range: the cumulative log decay inside a chunk is clamped at -80 so that 1/E_s stays finite in fp32; a key
-// channel that decays by more than e^-80 within 16 tokens is finite but no longer exact (the sequential kernel
-// has no such limit).
+// Range: a key channel whose total log decay over a 16-token chunk is below -80 gets its steps of that chunk scaled
+// to a total of -80, so that 1/E_s stays finite in fp32: finite and well ordered, but no longer exact for that channel
+// (a decay of e^-5 per token sustained over a whole chunk; RWKV-7 keeps d >= 0.54 per token, i.e. e^-10 per chunk).
+// The sequential kernels have no such limit.
 #include "chunk_common.h"
 #include "wkv_args.h"
 
@@ -139,6 +140,7 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
         if (F.nvalid != CK) l2 = valid ? l2 : 0.f;
         E[e] = row_scan(l2);
       }
+      cap_chunk_decay(E, lane);
     }
     if (slow) {
 #pragma unroll

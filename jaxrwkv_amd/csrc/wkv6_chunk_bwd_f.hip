@@ -14,7 +14,7 @@
 // 16q..16q+15, all 64 values, value x key accumulator tiles reused as B operands), 4 producer waves prepare the
 // state-independent operands into a ring of LDS slots; bounded-poll hand-shake.  The producers also own the terms
 // that need no state: u k c_t (handed over as an fp32 add-on) and du (summed per producer, combined at the end).
-// Range: the cumulative log decay inside a chunk is clamped at -80.
+// Range: as in the forward kernel, a chunk's total log decay per channel is capped at -80.
 #include "chunk_common.h"
 #include "wkv_args.h"
 
@@ -129,6 +129,7 @@ __device__ __forceinline__ void produce(Producer& P, const Raw& x, const ChunkFl
           if (F.nvalid != CK) l2 = valid ? l2 : 0.f;
           E[e] = row_scan(l2);
         }
+        cap_chunk_decay(E, lane);
       }
       if (slow) {
 #pragma unroll

@@ -15,7 +15,7 @@
 // rows of its 16 keys (all values, for G v) and G2 = the columns of its 16 values (all keys, for G^T k); both get the
 // same rank-16 update.  Products with fp32 quantities run as hi.hi + hi.lo + lo.hi on v_mfma_f32_16x16x32_bf16.
 // Work split, LDS ring and hand-shake as in the other chunked kernels; the producers also own the state-free terms
-// r u c_t and dy (r.(u k)), handed over as fp32 add-ons.  Range: cumulative log decay per chunk clamped at -80.
+// r u c_t and dy (r.(u k)), handed over as fp32 add-ons.  Range: a chunk's total log decay per channel is capped at -80.
 #include "chunk_common.h"
 #include "wkv_args.h"
 
@@ -137,6 +137,7 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
           if (F.nvalid != CK) l2 = valid ? l2 : 0.f;
           E[e] = row_scan(l2);
         }
+        cap_chunk_decay(E, lane);
       }
       if (slow) {
 #pragma unroll

@@ -39,9 +39,10 @@
 // The one chunk that holds token length-1 uses a second, masked operand set: for the state snapshot in the
 // forward pass, for the entry of the returned state's cotangent in the reverse sweep.
 //
-// Range: the cumulative log decay inside a chunk is clamped at -80 so that 1/E_s stays finite in fp32.  A key
-// channel whose decay over at most 16 tokens falls below e^-80 (RWKV-7 models keep d >= 0.54 per token, i.e.
-// e^-10 per chunk) is finite but no longer exact; the sequential kernels have no such limit.
+// Range: a key channel whose total log decay over a 16-token chunk is below -80 gets its steps of that chunk scaled
+// to a total of -80, so that 1/E_s stays finite in fp32: finite and well ordered, but no longer exact for that channel
+// (a decay of e^-5 per token sustained over a whole chunk; RWKV-7 keeps d >= 0.54 per token, i.e. e^-10 per chunk).
+// The sequential kernels have no such limit.
 #include "chunk_common.h"
 #include "wkv_args.h"
 
@@ -200,6 +201,7 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
       }
 #pragma unroll
       for (int e = 0; e < 8; ++e) E[e] = row_scan(fw[e]);
+      cap_chunk_decay(E, lane);
     }
     unpack8(x.a[hf], fa);
     if (slow) {

@@ -18,7 +18,7 @@
 // scaled operands, transposes, Gram tiles) into a ring of LDS slots; bounded-poll hand-shake.
 // new_starts inside a chunk restart the cumulative decay and mask the tiles; the chunk holding token length-1
 // also evaluates <dS_out, S_{length-1}> with a second, masked set of update operands.
-// Range: as in the forward kernel the cumulative log decay inside a chunk is clamped at -80.
+// Range: as in the forward kernel, a chunk's total log decay per channel is capped at -80.
 #include "chunk_common.h"
 #include "wkv_args.h"
 
@@ -160,6 +160,7 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
           if (F.nvalid != CK) l2 = valid ? l2 : 0.f;
           E[e] = row_scan(l2);
         }
+        cap_chunk_decay(E, lane);
       }
       if (slow) {
 #pragma unroll

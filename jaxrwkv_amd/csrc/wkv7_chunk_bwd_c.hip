@@ -19,7 +19,7 @@
 // as B operands), 4 producer waves prepare the state-independent operands into a ring of LDS slots; bounded-poll
 // hand-shake.  new_starts inside a chunk restart the cumulative decay and mask the tiles; the chunk holding token
 // length-1 adds the cotangent of the returned state through a second, masked set of row operands.
-// Range: the cumulative log decay inside a chunk is clamped at -80.
+// Range: as in the forward kernel, a chunk's total log decay per channel is capped at -80.
 #include "chunk_common.h"
 #include "wkv_args.h"
 
@@ -159,6 +159,7 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
           if (F.nvalid != CK) l2 = valid ? l2 : 0.f;
           E[e] = row_scan(l2);
         }
+        cap_chunk_decay(E, lane);
       }
       if (slow) {
 #pragma unroll
