@@ -1,0 +1,110 @@
+"""Size-independent properties at the full benchmark shapes (too large for the float64 oracle): the chunked MFMA
+kernels against the sequential fp32 kernels on the same inputs, a split call with the carried state against a
+single call, and a reset against a fresh run.  Comparisons stay on the GPU (torch) to keep the host out of it."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_rms(a, b):
+    a, b = a.float(), b.float()
+    return float((a - b).pow(2).mean().sqrt() / b.pow(2).mean().sqrt().clamp_min(1e-30))
+
+
+def wkv7_full(B=8, T=4096, H=32, N=64, seed=0):
+    g = torch.Generator("cuda").manual_seed(seed)
+    n = lambda *s: torch.randn(s, device="cuda", generator=g)
+    r, k, v, dy = (n(B, T, H, N).bfloat16() for _ in range(4))
+    w = (-0.5 + 0.5 * n(B, T, H, N)).bfloat16()
+    kap = torch.nn.functional.normalize(n(B, T, H, N), dim=-1)
+    a, b = (-kap).bfloat16(), (kap * torch.sigmoid(n(B, T, H, N))).bfloat16()
+    s = 0.1 * n(B, H, N, N)
+    ns = torch.rand((B, T), device="cuda", generator=g) < 1.0 / 1024
+    length = torch.randint(T // 2, T + 1, (B,), device="cuda", generator=g, dtype=torch.int32)
+    return dict(r=r, w=w, k=k, v=v, a=a, b=b, s=s, ns=ns, length=length, dy=dy)
+
+
+def test_wkv7_forward_and_backward_chunked_equals_sequential_at_the_headline_shape():
+    from jaxrwkv_amd import ops
+    x = wkv7_full()
+    args = (x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], x["length"], x["ns"])
+    ds = torch.randn_like(x["s"])
+    out = {}
+    for fs in (False, True):
+        new_s, y, sa = ops.wkv7_fwd(*args, compat=True, want_sa=True, force_seq=fs)
+        g = ops.wkv7_bwd(*args, x["dy"], sa, ds, compat=True, force_seq=fs)
+        out[fs] = (new_s, y, sa) + tuple(g)
+    torch.cuda.synchronize()
+    names = ("new_s", "y", "sa", "gr", "gw", "gk", "gv", "ga", "gb", "gs")
+    # bf16 outputs differ by their rounding (rel-rms 2^-9 ~ 2e-3 each side); fp32 ones by the hi+lo operand precision
+    tol = dict(new_s=2e-5, y=4e-3, sa=1e-4, gr=4e-3, gw=6e-3, gk=4e-3, gv=4e-3, ga=4e-3, gb=4e-3, gs=1e-4)
+    for n_, c, q in zip(names, out[False], out[True]):
+        assert torch.isfinite(c.float()).all(), n_
+        assert rel_rms(c, q) < tol[n_], (n_, rel_rms(c, q))
+
+
+def test_wkv7_split_call_with_carried_state_equals_single_call_at_the_headline_shape():
+    from jaxrwkv_amd import ops
+    x = wkv7_full(seed=1)
+    full_s, full_y, _ = ops.wkv7_fwd(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], None, x["ns"], compat=False)
+    h = 2048                                           # a multiple of the chunk length: identical chunking
+    sl = lambda t, a, b: t[:, a:b].contiguous()
+    s1, y1, _ = ops.wkv7_fwd(*(sl(x[n], 0, h) for n in "rwkvab"), x["s"], None, sl(x["ns"], 0, h), compat=False)
+    s2, y2, _ = ops.wkv7_fwd(*(sl(x[n], h, 4096) for n in "rwkvab"), s1, None, sl(x["ns"], h, 4096), compat=False)
+    torch.cuda.synchronize()
+    assert torch.equal(torch.cat([y1, y2], 1), full_y)
+    assert torch.equal(s2, full_s)
+
+
+def test_wkv7_reset_equals_fresh_run_at_the_headline_shape():
+    from jaxrwkv_amd import ops
+    x = wkv7_full(seed=2)
+    ns = torch.zeros_like(x["ns"])
+    ns[:, 2048] = True
+    _, y, _ = ops.wkv7_fwd(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], None, ns, compat=False)
+    sl = lambda t: t[:, 2048:].contiguous()
+    _, y2, _ = ops.wkv7_fwd(*(sl(x[n]) for n in "rwkvab"), torch.zeros_like(x["s"]), None, None, compat=False)
+    torch.cuda.synchronize()
+    assert torch.equal(y[:, 2048:], y2)
+
+
+def test_wkv6_chunked_equals_sequential_at_the_benchmark_shape():
+    from jaxrwkv_amd import ops
+    B, T, H, N = 16, 2048, 32, 64
+    g = torch.Generator("cuda").manual_seed(3)
+    n = lambda *s: torch.randn(s, device="cuda", generator=g)
+    r, k, v, dy = (n(B, T, H, N).bfloat16() for _ in range(4))
+    w = (-torch.exp(-0.5 + 0.5 * n(B, T, H, N))).bfloat16()
+    u = (0.5 * n(H, N)).bfloat16()
+    s = torch.zeros((B, H, N, N), device="cuda")
+    ns = torch.rand((B, T), device="cuda", generator=g) < 1.0 / 512
+    ds = n(B, H, N, N)
+    out = {}
+    for fs in (False, True):
+        new_s, y = ops.wkv6_fwd(r, k, v, w, u, s, None, ns, compat=True, force_seq=fs)
+        out[fs] = (new_s, y) + tuple(ops.wkv6_bwd(r, k, v, w, u, s, None, ns, dy, ds, compat=True, force_seq=fs))
+    torch.cuda.synchronize()
+    names = ("new_s", "y", "gr", "gk", "gv", "gw", "gu", "gs")
+    tol = dict(new_s=2e-5, y=4e-3, gr=4e-3, gk=4e-3, gv=4e-3, gw=6e-3, gu=4e-3, gs=1e-4)
+    for n_, c, q in zip(names, out[False], out[True]):
+        assert torch.isfinite(c.float()).all(), n_
+        assert rel_rms(c, q) < tol[n_], (n_, rel_rms(c, q))
+
+
+def test_wkv4_split_call_equals_single_call_at_the_benchmark_shape():
+    from jaxrwkv_amd import ops
+    B, T, C = 32, 4096, 2560
+    g = torch.Generator("cuda").manual_seed(4)
+    k = torch.randn((B, T, C), device="cuda", generator=g)
+    v = torch.randn((B, T, C), device="cuda", generator=g)
+    w = -torch.exp(torch.randn(C, device="cuda", generator=g))
+    u = 0.5 * torch.randn(C, device="cuda", generator=g)
+    s = torch.zeros((B, 3, C), device="cuda")
+    s[:, 2] = -1e38
+    full_s, full_y = ops.wkv4_fwd(w, u, k, v, s, None, None, compat=False)
+    s1, y1 = ops.wkv4_fwd(w, u, k[:, :1000].contiguous(), v[:, :1000].contiguous(), s, None, None, compat=False)
+    s2, y2 = ops.wkv4_fwd(w, u, k[:, 1000:].contiguous(), v[:, 1000:].contiguous(), s1, None, None, compat=False)
+    torch.cuda.synchronize()
+    assert torch.equal(torch.cat([y1, y2], 1), full_y)
+    assert torch.equal(s2, full_s)
