@@ -132,6 +132,19 @@ int hiprwkv_wkv4_bwd(hiprwkv_stream stream, int io_dtype,
                      float* gw, float* gu, void* gk, void* gv, void* gs,
                      void* workspace, size_t workspace_bytes, unsigned flags);
 
+/* ---- RWKV-7 time-mixing stages around the op (forward only) -------------------------
+ * The element-wise work the reference does in jnp on either side of inner_loop (rwkv7.py:248-252, 257 and :263-265),
+ * fused into one pass each; it has no counterpart among the reference's ffi targets.  `rows` = number of tokens
+ * (all batch axes flattened), tensors (rows, H, 64) io_dtype, parameters k_k, k_a, ln_w, ln_b, r_k (H, 64) io_dtype.
+ *   premix : kk = normalize_head(k . k_k); k_out = k (1 + (a - 1) k_a); a_out = -kk; b_out = kk . a
+ *   postmix: out = (group_norm_head(y, eps) . ln_w + ln_b + (sum_j r_j k_j r_k_j) v) . g      (k = premix's k_out) */
+int hiprwkv_rwkv7_premix(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t H, int64_t N,
+                         const void* k, const void* a, const void* k_k, const void* k_a,
+                         void* k_out, void* a_out, void* b_out);
+int hiprwkv_rwkv7_postmix(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t H, int64_t N,
+                          const void* y, const void* r, const void* k, const void* v, const void* g,
+                          const void* ln_w, const void* ln_b, const void* r_k, float eps, void* out);
+
 #ifdef __cplusplus
 }
 #endif

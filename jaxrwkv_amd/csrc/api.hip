@@ -240,4 +240,33 @@ int hiprwkv_wkv4_bwd(hiprwkv_stream stream, int io_dtype, int64_t B, int64_t T, 
   return HIPRWKV_OK;
 }
 
+int hiprwkv_rwkv7_premix(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t H, int64_t N, const void* k,
+                         const void* a, const void* k_k, const void* k_a, void* k_out, void* a_out, void* b_out) {
+  if (!dtype_ok(io_dtype)) return fail(HIPRWKV_EINVAL, "rwkv7_premix: dtype must be HIPRWKV_F32 or HIPRWKV_BF16");
+  if (N != 64) return fail(HIPRWKV_EINVAL, "rwkv7_premix: head size N=%lld not supported (64 only)", (long long)N);
+  if (rows <= 0 || H <= 0 || (rows * H + 3) / 4 > 0x7fffffffLL) return fail(HIPRWKV_EINVAL, "rwkv7_premix: bad rows/H");
+  const void* req[] = {k, a, k_k, k_a, k_out, a_out, b_out};
+  for (const void* p : req)
+    if (p == nullptr) return fail(HIPRWKV_EINVAL, "rwkv7_premix: null tensor pointer");
+  hipError_t e = launch_rwkv7_premix(io_dtype == HIPRWKV_F32, rows, H, k, a, k_k, k_a, k_out, a_out, b_out,
+                                     static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "rwkv7_premix: %s", hipGetErrorString(e));
+  return HIPRWKV_OK;
+}
+
+int hiprwkv_rwkv7_postmix(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t H, int64_t N, const void* y,
+                          const void* r, const void* k, const void* v, const void* g, const void* ln_w,
+                          const void* ln_b, const void* r_k, float eps, void* out) {
+  if (!dtype_ok(io_dtype)) return fail(HIPRWKV_EINVAL, "rwkv7_postmix: dtype must be HIPRWKV_F32 or HIPRWKV_BF16");
+  if (N != 64) return fail(HIPRWKV_EINVAL, "rwkv7_postmix: head size N=%lld not supported (64 only)", (long long)N);
+  if (rows <= 0 || H <= 0 || (rows * H + 3) / 4 > 0x7fffffffLL) return fail(HIPRWKV_EINVAL, "rwkv7_postmix: bad rows/H");
+  const void* req[] = {y, r, k, v, g, ln_w, ln_b, r_k, out};
+  for (const void* p : req)
+    if (p == nullptr) return fail(HIPRWKV_EINVAL, "rwkv7_postmix: null tensor pointer");
+  hipError_t e = launch_rwkv7_postmix(io_dtype == HIPRWKV_F32, rows, H, y, r, k, v, g, ln_w, ln_b, r_k, eps, out,
+                                      static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "rwkv7_postmix: %s", hipGetErrorString(e));
+  return HIPRWKV_OK;
+}
+
 }  // extern "C"

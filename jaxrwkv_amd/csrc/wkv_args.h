@@ -74,5 +74,10 @@ hipError_t launch_wkv6_chunk_bwd_f(const Wkv6Args& A, hipStream_t stream);
 hipError_t launch_wkv6_chunk_bwd_r(const Wkv6Args& A, hipStream_t stream);
 hipError_t launch_wkv4_fwd(const Wkv4Args& A, hipStream_t stream);
 hipError_t launch_wkv4_bwd(const Wkv4Args& A, hipStream_t stream);
+hipError_t launch_rwkv7_premix(int io_f32, int64_t rows, int64_t H, const void* k, const void* a, const void* k_k,
+                               const void* k_a, void* k_out, void* a_out, void* b_out, hipStream_t stream);
+hipError_t launch_rwkv7_postmix(int io_f32, int64_t rows, int64_t H, const void* y, const void* r, const void* k,
+                                const void* v, const void* g, const void* ln_w, const void* ln_b, const void* r_k,
+                                float eps, void* out, hipStream_t stream);
 
 }  // namespace hiprwkv

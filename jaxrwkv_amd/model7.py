@@ -17,6 +17,7 @@ import math
 import torch
 import torch.nn.functional as F
 
+from . import ops
 from .rwkv7 import HipRWKV
 
 HEAD_SIZE = 64
@@ -115,6 +116,8 @@ class RWKV7:
     """``forward`` / ``default_state`` with the reference's argument names; batched over the leading axis."""
 
     inner = HipRWKV
+    #: use the fused pre/post time-mixing kernels (ops.rwkv7_premix / rwkv7_postmix) when no gradient is recorded
+    fuse_mix = True
 
     @classmethod
     def default_state(cls, params, batch):
@@ -155,19 +158,28 @@ class RWKV7:
             v = v + (v_first - v) * torch.sigmoid(att["v0"] + (xv @ att["v1"]) @ att["v2"])
         a = torch.sigmoid(att["a0"] + (xa @ att["a1"]) @ att["a2"])
         g = torch.sigmoid(xg @ att["g1"]) @ att["g2"]
-        kk = (k * att["k_k"]).reshape(B, T, H, N)
-        kk = (kk / torch.clamp(torch.linalg.vector_norm(kk.float(), dim=-1, keepdim=True), min=1e-12).to(kk.dtype))
-        kk = kk.reshape(B, T, C)
-        k = k * (1 + (a - 1) * att["k_a"])
         new_shift = x[torch.arange(B, device=x.device), last_idx]
         s = wkv_state.reshape(B, H, N, N)
-        rh, wh, kh, vh, ah, bh = (t.reshape(B, T, H, N) for t in (r, w, k, v, -kk, kk * a))
+        fused = cls.fuse_mix and not torch.is_grad_enabled()      # the fused stages have no backward
+        rh, wh, vh = (t.reshape(B, T, H, N) for t in (r, w, v))
+        if fused:
+            kh, ah, bh = ops.rwkv7_premix(k.reshape(B, T, H, N), a.reshape(B, T, H, N), att["k_k"], att["k_a"])
+        else:
+            kk = (k * att["k_k"]).reshape(B, T, H, N)
+            kk = (kk / torch.clamp(torch.linalg.vector_norm(kk.float(), dim=-1, keepdim=True), min=1e-12).to(kk.dtype))
+            kk = kk.reshape(B, T, C)
+            k = k * (1 + (a - 1) * att["k_a"])
+            kh, ah, bh = (t.reshape(B, T, H, N) for t in (k, -kk, kk * a))
         s_new, out = cls.inner.inner_loop(rh, wh, kh, vh, ah, bh, s, length, new_starts)
-        y = out.reshape(B * T, H, N).float()
-        y = F.group_norm(y.reshape(B * T, C), H, att["ln_x"]["weight"].float(), att["ln_x"]["bias"].float(), 64e-5)
-        y = y.to(x.dtype).reshape(B, T, C)
-        bonus = ((rh * kh * att["r_k"]).sum(-1, keepdim=True) * vh).reshape(B, T, C)
-        y = (y + bonus) * g
+        if fused:
+            y = ops.rwkv7_postmix(out, rh, kh, vh, g.reshape(B, T, H, N), att["ln_x"]["weight"], att["ln_x"]["bias"],
+                                  att["r_k"], 64e-5).reshape(B, T, C)
+        else:
+            y = out.reshape(B * T, H, N).float()
+            y = F.group_norm(y.reshape(B * T, C), H, att["ln_x"]["weight"].float(), att["ln_x"]["bias"].float(), 64e-5)
+            y = y.to(x.dtype).reshape(B, T, C)
+            bonus = ((rh * kh * att["r_k"]).sum(-1, keepdim=True) * vh).reshape(B, T, C)
+            y = (y + bonus) * g
         return y @ att["output"]["weight"].T, new_shift, s_new.reshape(B, N, C), v_first
 
     @classmethod

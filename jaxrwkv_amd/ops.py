@@ -259,3 +259,36 @@ def wkv4(w_neg, u, k, v, s, length=None, new_starts=None, compat=True):
     B, T = k.shape[:2]
     length, new_starts = _length_ns(length, new_starts, B, T, k.device)
     return _Wkv4.apply(w_neg, u, k, v, s, length, new_starts, compat)
+
+
+# ----------------------------------------------------------------------------- RWKV-7 time-mixing stages (forward only)
+def rwkv7_premix(k, a, k_k, k_a):
+    """k, a (..., H, N); k_k, k_a (H, N).  Returns (k', a_i, b_i) of rwkv7.py:248-252, 257: kk = normalize_head(k k_k),
+    k' = k (1 + (a - 1) k_a), a_i = -kk, b_i = kk a.  No autograd: for inference paths."""
+    lib = _lib.load()
+    io = k.dtype
+    H, N = k.shape[-2:]
+    k, a = _dev(k, io), _dev(a, io)
+    k_k, k_a = _dev(k_k.reshape(H, N), io), _dev(k_a.reshape(H, N), io)
+    rows = k.numel() // (H * N)
+    k_out, a_out, b_out = (torch.empty_like(k) for _ in range(3))
+    rc = lib.hiprwkv_rwkv7_premix(_stream(), _DT[io], rows, H, N, _p(k), _p(a), _p(k_k), _p(k_a), _p(k_out), _p(a_out),
+                                  _p(b_out))
+    _lib.check(rc, "hiprwkv_rwkv7_premix")
+    return k_out, a_out, b_out
+
+
+def rwkv7_postmix(y, r, k, v, g, ln_w, ln_b, r_k, eps=64e-5):
+    """y, r, k, v, g (..., H, N); ln_w, ln_b, r_k (H, N).  Returns (group_norm_head(y) ln_w + ln_b + (r.k.r_k) v) g of
+    rwkv7.py:263-265.  No autograd: for inference paths."""
+    lib = _lib.load()
+    io = y.dtype
+    H, N = y.shape[-2:]
+    y, r, k, v, g = (_dev(x, io) for x in (y, r, k, v, g))
+    ln_w, ln_b, r_k = (_dev(x.reshape(H, N), io) for x in (ln_w, ln_b, r_k))
+    rows = y.numel() // (H * N)
+    out = torch.empty_like(y)
+    rc = lib.hiprwkv_rwkv7_postmix(_stream(), _DT[io], rows, H, N, _p(y), _p(r), _p(k), _p(v), _p(g), _p(ln_w), _p(ln_b),
+                                   _p(r_k), float(eps), _p(out))
+    _lib.check(rc, "hiprwkv_rwkv7_postmix")
+    return out

@@ -104,3 +104,45 @@ def test_decode_step_in_a_hip_graph_replays_like_eager():
         assert torch.equal(g_logits, e_logits), it
         assert torch.equal(g_state, e_state), it
         state.copy_(e_state)                          # carry the state into the next step
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_fused_time_mixing_stages_against_torch_fp32(dtype):
+    """ops.rwkv7_premix / rwkv7_postmix against plain torch fp32 of rwkv7.py:248-252, 257, 263-265."""
+    from jaxrwkv_amd import ops
+    g = torch.Generator("cuda").manual_seed(9)
+    B, T, H, N = 2, 37, 3, 64
+    n = lambda *s: torch.randn(s, device="cuda", generator=g).to(dtype)
+    k, y, r, v, gate = n(B, T, H, N), n(B, T, H, N), n(B, T, H, N), n(B, T, H, N), n(B, T, H, N)
+    a = torch.sigmoid(n(B, T, H, N).float()).to(dtype)
+    k_k, k_a, lnw, lnb, r_k = n(H, N), n(H, N), n(H, N), n(H, N), n(H, N)
+    k2, ai, bi = ops.rwkv7_premix(k, a, k_k, k_a)
+    f = lambda t: t.float()
+    kk = f(k) * f(k_k)
+    kk = kk / torch.clamp(torch.linalg.vector_norm(kk, dim=-1, keepdim=True), min=1e-12)
+    tol = dict(rtol=1e-5, atol=1e-6) if dtype == torch.float32 else dict(rtol=2.0 ** -7, atol=1e-6)
+    torch.testing.assert_close(f(k2), f(k) * (1 + (f(a) - 1) * f(k_a)), **tol)
+    torch.testing.assert_close(f(ai), -kk, **tol)
+    torch.testing.assert_close(f(bi), kk * f(a), **tol)
+    out = ops.rwkv7_postmix(y, r, k2, v, gate, lnw, lnb, r_k, 64e-5)
+    yf = f(y)
+    yn = (yf - yf.mean(-1, keepdim=True)) / torch.sqrt(yf.var(-1, unbiased=False, keepdim=True) + 64e-5) * f(lnw) + f(lnb)
+    ref = (yn + (f(r) * f(k2) * f(r_k)).sum(-1, keepdim=True) * f(v)) * f(gate)
+    tol = dict(rtol=1e-4, atol=1e-4) if dtype == torch.float32 else dict(rtol=2.0 ** -7, atol=2e-2)
+    torch.testing.assert_close(f(out), ref, **tol)
+
+
+def test_model_with_and_without_fused_stages_agree():
+    from jaxrwkv_amd.model7 import RWKV7, randomize_weights
+    params = randomize_weights(13, 2, 128, 211, dtype=torch.float32, device="cuda", zero_init=False)
+    tok = torch.randint(0, 211, (2, 33), device="cuda", generator=torch.Generator("cuda").manual_seed(1))
+    state = RWKV7.default_state(params, 2)
+    with torch.no_grad():
+        a = RWKV7.forward(params, tok, state)
+        RWKV7.fuse_mix = False
+        try:
+            b = RWKV7.forward(params, tok, state)
+        finally:
+            RWKV7.fuse_mix = True
+    torch.testing.assert_close(a[0], b[0], rtol=1e-4, atol=1e-4)
+    torch.testing.assert_close(a[1], b[1], rtol=1e-4, atol=1e-4)
