@@ -61,10 +61,12 @@ __device__ __forceinline__ void split2(float x0, float x1, uint32_t& hi, uint32_
   hi = __builtin_amdgcn_perm(__float_as_uint(x1), __float_as_uint(x0), 0x07060302u);
   // x - hi in one v_dot2c_f32_bf16 each: acc += hi.lo * -1 + hi.hi * 0  (resp. 0, -1)
   // The two selectors are kept out of the compiler's sight: written as immediates, (-1, 0) would be encoded as
-  // the 16-bit inline constant -1.0, whose bit pattern is the fp16 one.
+  // the 16-bit inline constant -1.0, whose bit pattern is the fp16 one.  The asm statements are not volatile, so
+  // that the selectors are materialised once per kernel, not once per call.
   const bf16x2_t hp = __builtin_bit_cast(bf16x2_t, hi);
   uint32_t m10 = 0x0000bf80u, m01 = 0xbf800000u;
-  asm volatile("" : "+s"(m10), "+s"(m01));
+  asm("" : "+s"(m10));
+  asm("" : "+s"(m01));
   const float l0 = __builtin_amdgcn_fdot2_f32_bf16(hp, __builtin_bit_cast(bf16x2_t, m10), x0, false);
   const float l1 = __builtin_amdgcn_fdot2_f32_bf16(hp, __builtin_bit_cast(bf16x2_t, m01), x1, false);
   lo = pack_rn(l0, l1);
