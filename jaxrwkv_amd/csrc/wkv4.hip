@@ -6,95 +6,152 @@
 //     ww = pp + w  ; q = max(ww, k_t) ; aa = e^{ww-q} aa + e^{k_t-q} v_t ; bb = e^{ww-q} bb + e^{k_t-q} ; pp = q
 // In each pair of exponentials one argument is exactly 0, so a step costs two exp, not four.
 // k and v are streamed with a register prefetch of TB steps per thread (coalesced across channels), which keeps
-// enough bytes in flight to cover HBM latency with the few waves per CU this problem has.
+// enough bytes in flight to cover HBM latency with the few waves per CU this problem has.  A lone wave issues one
+// instruction every ~4.6 cycles whatever its kind, so the step is kept short: blocks of TB steps without a reset,
+// a sequence end or the token length-1 run a loop without per-step checks, the reset flags of a block are fetched
+// by one load (a byte per lane, one block ahead) and turned into a uniform mask, and the quotient is num * rcp(den)
+// (v_rcp_f32 is good to 1 ulp; the reference divides, the difference is ~1e-7 relative).
 #include "common.h"
 #include "wkv_args.h"
 
 namespace hiprwkv {
 
 constexpr int W4_THREADS = 64;
-constexpr int W4_TB = 16;
+constexpr int W4_TB = 32;
 constexpr float W4_RESET_PP = -1e30f;  // rwkv4.py:149-150
+
+namespace {
+
+// y_t from the state entering step t, then the state after it
+__device__ __forceinline__ float wkv4_step(float& aa, float& bb, float& pp, float kt, float vt, float w, float u) {
+  float y;
+  {
+    const float diff = pp - (u + kt);                  // e1 = e^{pp-q}, e2 = e^{ww-q}
+    const float e = __expf(-fabsf(diff));
+    const float e1 = diff >= 0.f ? 1.f : e;
+    const float e2 = diff >= 0.f ? e : 1.f;
+    const float num = fmaf(e1, aa, e2 * vt);
+    const float den = fmaf(e1, bb, e2);
+    y = num * __builtin_amdgcn_rcpf(den);
+  }
+  {
+    const float ww = pp + w;
+    const float diff = ww - kt;                        // e1 = e^{ww-q}, e2 = e^{k-q}
+    const float e = __expf(-fabsf(diff));
+    const float e1 = diff >= 0.f ? 1.f : e;
+    const float e2 = diff >= 0.f ? e : 1.f;
+    aa = fmaf(e1, aa, e2 * vt);
+    bb = fmaf(e1, bb, e2);
+    pp = fmaxf(ww, kt);
+  }
+  return y;
+}
+
+// Raw buffer access: address = descriptor base (scalar) + lane offset (one VGPR, loop-invariant) + scalar offset.
+// Stepping through the tokens then costs one scalar add for k, v and y together, and no vector address arithmetic.
+using rsrc_t = __amdgpu_buffer_rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void* base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7fffffff, 0x00020000);
+}
+__device__ __forceinline__ float buf_ld(const float*, rsrc_t r, int voff, int soff) {
+  return __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+}
+__device__ __forceinline__ float buf_ld(const bf16_t*, rsrc_t r, int voff, int soff) {
+  return bf16_to_f32(__builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, 0));
+}
+__device__ __forceinline__ void buf_st(float*, float x, rsrc_t r, int voff, int soff) {
+  __builtin_amdgcn_raw_buffer_store_b32(__float_as_uint(x), r, voff, soff, 0);
+}
+__device__ __forceinline__ void buf_st(bf16_t*, float x, rsrc_t r, int voff, int soff) {
+  __builtin_amdgcn_raw_buffer_store_b16(f32_to_bf16(x), r, voff, soff, 0);
+}
+
+}  // namespace
 
 template <typename IO>
 __global__ __launch_bounds__(W4_THREADS) void wkv4_fwd_kernel(Wkv4Args A) {
+  static_assert(W4_TB <= W4_THREADS, "one lane per reset flag of a block");
   const int64_t cblocks = (A.C + W4_THREADS - 1) / W4_THREADS;
   const int64_t b = blockIdx.x / cblocks;
   const int64_t c = (blockIdx.x % cblocks) * W4_THREADS + threadIdx.x;
-  if (c >= A.C) return;
-  const IO* kp = reinterpret_cast<const IO*>(A.k) + (size_t)b * A.T * A.C + c;
-  const IO* vp = reinterpret_cast<const IO*>(A.v) + (size_t)b * A.T * A.C + c;
-  IO* yp = reinterpret_cast<IO*>(A.out) + (size_t)b * A.T * A.C + c;
-  const IO* sp = reinterpret_cast<const IO*>(A.s) + (size_t)b * 3 * A.C + c;
-  IO* nsp = reinterpret_cast<IO*>(A.new_s) + (size_t)b * 3 * A.C + c;
+  // lanes beyond C work on channel C-1 as well: they load the same values and store the same results to the same
+  // places as that channel's own lane, so no access needs a predicate
+  const int64_t cc = c < A.C ? c : A.C - 1;
+  const IO* kseq = reinterpret_cast<const IO*>(A.k) + (size_t)b * A.T * A.C;
+  const IO* vseq = reinterpret_cast<const IO*>(A.v) + (size_t)b * A.T * A.C;
+  IO* yseq = reinterpret_cast<IO*>(A.out) + (size_t)b * A.T * A.C;
+  const IO* sp = reinterpret_cast<const IO*>(A.s) + (size_t)b * 3 * A.C + cc;
+  IO* nsp = reinterpret_cast<IO*>(A.new_s) + (size_t)b * 3 * A.C + cc;
   const uint8_t* ns = A.ns ? A.ns + (size_t)b * A.T : nullptr;
-  const float w = ld_f(reinterpret_cast<const IO*>(A.w) + c);
-  const float u = ld_f(reinterpret_cast<const IO*>(A.u) + c);
+  const float w = ld_f(reinterpret_cast<const IO*>(A.w) + cc);
+  const float u = ld_f(reinterpret_cast<const IO*>(A.u) + cc);
   float aa = ld_f(sp), bb = ld_f(sp + A.C), pp = ld_f(sp + 2 * A.C);
   int64_t L = A.length ? (int64_t)A.length[b] : A.T;
   L = L < A.T ? L : A.T;
   const bool q2drop = (A.flags & 1u) && L < A.T && ns != nullptr && ns[L] != 0;
-  if (L == 0) {
+  auto snapshot = [&]() {
     st_f(nsp, q2drop ? 0.f : aa);
     st_f(nsp + A.C, q2drop ? 0.f : bb);
     st_f(nsp + 2 * A.C, q2drop ? W4_RESET_PP : pp);
-  }
+  };
+  if (L == 0) snapshot();
 
+  const int lane = threadIdx.x;
+  const int voff = (int)(cc * sizeof(IO));
+  const int stride = (int)(A.C * sizeof(IO));        // bytes between consecutive tokens
   float kb[W4_TB], vb[W4_TB];
+  uint8_t nsb = 0;                                    // this lane's reset flag of the block after the current one
   auto fetch = [&](int64_t t0) {
+    const rsrc_t rk = make_rsrc(kseq + (size_t)t0 * A.C), rv = make_rsrc(vseq + (size_t)t0 * A.C);
+    int soff = 0;
+    if (t0 + W4_TB <= A.T) {
 #pragma unroll
-    for (int x = 0; x < W4_TB; ++x) {
-      const int64_t t = t0 + x;
-      if (t < A.T) {
-        kb[x] = ld_f(kp + (size_t)t * A.C);
-        vb[x] = ld_f(vp + (size_t)t * A.C);
-      } else {
-        kb[x] = 0.f;
-        vb[x] = 0.f;
+      for (int x = 0; x < W4_TB; ++x) {
+        kb[x] = buf_ld(kseq, rk, voff, soff);
+        vb[x] = buf_ld(vseq, rv, voff, soff);
+        soff += stride;
+      }
+    } else {
+#pragma unroll
+      for (int x = 0; x < W4_TB; ++x) {
+        const bool in = t0 + x < A.T;
+        kb[x] = in ? buf_ld(kseq, rk, voff, soff) : 0.f;
+        vb[x] = in ? buf_ld(vseq, rv, voff, soff) : 0.f;
+        soff += stride;
       }
     }
+    nsb = 0;
+    if (ns != nullptr && lane < W4_TB && t0 + lane < A.T) nsb = ns[t0 + lane];
   };
   fetch(0);
   for (int64_t t0 = 0; t0 < A.T; t0 += W4_TB) {
     float kc[W4_TB], vc[W4_TB];
-    uint32_t rmask = 0;
 #pragma unroll
     for (int x = 0; x < W4_TB; ++x) {
       kc[x] = kb[x];
       vc[x] = vb[x];
-      if (ns != nullptr && t0 + x < A.T && ns[t0 + x]) rmask |= 1u << x;
     }
+    const uint64_t rmask = ns != nullptr ? __ballot(nsb != 0) : 0ull;
     if (t0 + W4_TB < A.T) fetch(t0 + W4_TB);
+    const rsrc_t ry = make_rsrc(yseq + (size_t)t0 * A.C);
+    int soff = 0;
+    const bool plain = rmask == 0ull && t0 + W4_TB <= A.T && (L - 1 < t0 || L - 1 >= t0 + W4_TB);
+    if (plain) {
 #pragma unroll
-    for (int x = 0; x < W4_TB; ++x) {
-      const int64_t t = t0 + x;
-      if (t < A.T) {
-      if (rmask & (1u << x)) { aa = 0.f; bb = 0.f; pp = W4_RESET_PP; }
-      const float kt = kc[x], vt = vc[x];
-      {
-        const float diff = pp - (u + kt);                  // e1 = e^{pp-q}, e2 = e^{ww-q}
-        const float e = __expf(-fabsf(diff));
-        const float e1 = diff >= 0.f ? 1.f : e;
-        const float e2 = diff >= 0.f ? e : 1.f;
-        const float num = fmaf(e1, aa, e2 * vt);
-        const float den = fmaf(e1, bb, e2);
-        st_f(yp + (size_t)t * A.C, __fdividef(num, den));
+      for (int x = 0; x < W4_TB; ++x) {
+        buf_st(yseq, wkv4_step(aa, bb, pp, kc[x], vc[x], w, u), ry, voff, soff);
+        soff += stride;
       }
-      {
-        const float ww = pp + w;
-        const float diff = ww - kt;                        // e1 = e^{ww-q}, e2 = e^{k-q}
-        const float e = __expf(-fabsf(diff));
-        const float e1 = diff >= 0.f ? 1.f : e;
-        const float e2 = diff >= 0.f ? e : 1.f;
-        aa = fmaf(e1, aa, e2 * vt);
-        bb = fmaf(e1, bb, e2);
-        pp = fmaxf(ww, kt);
-      }
-      if (t == L - 1) {
-        st_f(nsp, q2drop ? 0.f : aa);
-        st_f(nsp + A.C, q2drop ? 0.f : bb);
-        st_f(nsp + 2 * A.C, q2drop ? W4_RESET_PP : pp);
-      }
+    } else {
+#pragma unroll
+      for (int x = 0; x < W4_TB; ++x) {
+        const int64_t t = t0 + x;
+        if (t < A.T) {
+          if (rmask & (1ull << x)) { aa = 0.f; bb = 0.f; pp = W4_RESET_PP; }
+          buf_st(yseq, wkv4_step(aa, bb, pp, kc[x], vc[x], w, u), ry, voff, soff);
+          if (t == L - 1) snapshot();
+        }
+        soff += stride;
       }
     }
   }
@@ -192,7 +249,7 @@ __global__ __launch_bounds__(W4_THREADS) void wkv4_bwd_kernel(Wkv4Args A) {
     // states entering each step of the segment
 #pragma unroll
     for (int x = 0; x < W4_SEG; ++x) {
-      if (rmask & (1u << x)) { aa = 0.f; bb = 0.f; pp = W4_RESET_PP; }
+      if (rmask & (1ull << x)) { aa = 0.f; bb = 0.f; pp = W4_RESET_PP; }
       sa[x] = aa; sb[x] = bb; spp[x] = pp;
       const float ww = pp + w, diff = ww - kc[x];
       const float e = __expf(-fabsf(diff));
