@@ -341,16 +341,23 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
   }
   // outputs: register i is token 4g+i, lanes n = 16 consecutive keys
   const size_t lo = (size_t)oc.voff;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  auto put = [&](int i, bool full) {
     const int tok = 4 * g + i;
     const float sdy = (P[i] + P2[i]) * slot->Ee[tok][16 * q + n];
     const float rr = bf16_to_f32(slot->R[tok][16 * q + n]);
     const float ukc = slot->UKC[tok][16 * q + n];
-    if (tok < nvalid) {
+    if (full || tok < nvalid) {
       *reinterpret_cast<uint16_t*>(oc.gr + lo * 2 + i * oc.tok_bytes) = f32_to_bf16(ukc + sdy);
       *reinterpret_cast<float*>(oc.er + lo * 4 + 2 * i * oc.tok_bytes) = rr * sdy;
     }
+  };
+  if (nvalid == CK) {      // every chunk but a partial last one: no per-lane predicates
+#pragma unroll
+    for (int i = 0; i < 4; ++i) put(i, true);
+  } else {
+    rare_path();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) put(i, false);
   }
   oc.gr += CK * oc.tok_bytes;
   oc.er += 2 * CK * oc.tok_bytes;

@@ -456,17 +456,24 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
     C.carry = cin;
   }
   const size_t lo = (size_t)cu.voff;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  auto put = [&](int i, bool full) {
     const int tok = 4 * g + i;
     const float dk = slot->RUC[tok][16 * q + n] + gvk[i];
     const float dv = slot->DYR[tok][16 * q + n] + PV[i] + PV2[i];
     const float dw = ((resets >> tok) & 1u) ? 0.f : cy[i] - pre.er[i];
-    if (tok < nvalid) {
+    if (full || tok < nvalid) {
       *reinterpret_cast<uint16_t*>(cu.gk + lo * 2 + i * cu.tok_bytes) = f32_to_bf16(dk);
       *reinterpret_cast<uint16_t*>(cu.gv + lo * 2 + i * cu.tok_bytes) = f32_to_bf16(dv);
       *reinterpret_cast<uint16_t*>(cu.gw + lo * 2 + i * cu.tok_bytes) = f32_to_bf16(dw);
     }
+  };
+  if (nvalid == CK) {      // every chunk but a partial last one: no per-lane predicates
+#pragma unroll
+    for (int i = 0; i < 4; ++i) put(i, true);
+  } else {
+    rare_path();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) put(i, false);
   }
 }
 

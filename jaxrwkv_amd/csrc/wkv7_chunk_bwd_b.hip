@@ -403,19 +403,26 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
 #pragma unroll
   for (int i = 0; i < 5; ++i) e[i] = slot->E[4 * g + i][16 * q + n];
   const size_t lo = (size_t)oc.voff;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  auto put = [&](int i, bool full) {
     const int tok = 4 * g + i;
     const float rr = bf16_to_f32(slot->RA[0][tok][16 * q + n]);
     const float aa = bf16_to_f32(slot->RA[1][tok][16 * q + n]);
     const float dr = DR[i] * e[i + 1];
     const float da = DA[i] * e[i];
-    if (tok < nvalid) {
+    if (full || tok < nvalid) {
       *reinterpret_cast<uint16_t*>(oc.gr + lo * 2 + i * oc.tok_bytes) = f32_to_bf16(dr);
       *reinterpret_cast<uint16_t*>(oc.ga + lo * 2 + i * oc.tok_bytes) = f32_to_bf16(da);
       *reinterpret_cast<float*>(oc.e2 + lo * 4 + 2 * i * oc.tok_bytes) = aa * da;
       *reinterpret_cast<float*>(oc.e3 + lo * 4 + 2 * i * oc.tok_bytes) = fmaf(rr, dr, tok == snap_tok ? inj : 0.f);
     }
+  };
+  if (nvalid == CK) {      // every chunk but a partial last one: no per-lane predicates
+#pragma unroll
+    for (int i = 0; i < 4; ++i) put(i, true);
+  } else {
+    rare_path();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) put(i, false);
   }
   oc.gr += CK * oc.tok_bytes; oc.ga += CK * oc.tok_bytes;
   oc.e2 += 2 * CK * oc.tok_bytes; oc.e3 += 2 * CK * oc.tok_bytes;

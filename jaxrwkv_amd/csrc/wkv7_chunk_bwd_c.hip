@@ -314,17 +314,26 @@ struct Cursor {
 
 __device__ __forceinline__ void prefetch(Pre& p, const Cursor& cu, int nvalid, int g) {
   const size_t lo = (size_t)cu.voff;
+  auto get = [&](int i) {
+    p.e2[i] = *reinterpret_cast<const float*>(cu.e2 + lo * 4 + 2 * i * cu.tok_bytes);
+    p.e3[i] = *reinterpret_cast<const float*>(cu.e3 + lo * 4 + 2 * i * cu.tok_bytes);
+    p.k[i] = *reinterpret_cast<const uint16_t*>(cu.k + lo * 2 + i * cu.tok_bytes);
+    p.b[i] = *reinterpret_cast<const uint16_t*>(cu.b + lo * 2 + i * cu.tok_bytes);
+    p.w[i] = *reinterpret_cast<const uint16_t*>(cu.w + lo * 2 + i * cu.tok_bytes);
+  };
+  if (nvalid == CK) {      // every chunk but a partial last one: no per-lane predicates
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    if (4 * g + i < nvalid) {
-      p.e2[i] = *reinterpret_cast<const float*>(cu.e2 + lo * 4 + 2 * i * cu.tok_bytes);
-      p.e3[i] = *reinterpret_cast<const float*>(cu.e3 + lo * 4 + 2 * i * cu.tok_bytes);
-      p.k[i] = *reinterpret_cast<const uint16_t*>(cu.k + lo * 2 + i * cu.tok_bytes);
-      p.b[i] = *reinterpret_cast<const uint16_t*>(cu.b + lo * 2 + i * cu.tok_bytes);
-      p.w[i] = *reinterpret_cast<const uint16_t*>(cu.w + lo * 2 + i * cu.tok_bytes);
-    } else {
-      p.e2[i] = p.e3[i] = 0.f;
-      p.k[i] = p.b[i] = p.w[i] = 0;
+    for (int i = 0; i < 4; ++i) get(i);
+  } else {
+    rare_path();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (4 * g + i < nvalid) {
+        get(i);
+      } else {
+        p.e2[i] = p.e3[i] = 0.f;
+        p.k[i] = p.b[i] = p.w[i] = 0;
+      }
     }
   }
 }
@@ -459,16 +468,23 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
     C.carry = cin;
   }
   const size_t lo = (size_t)cu.voff;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  auto put = [&](int i, bool full) {
     const int tok = 4 * g + i;
-    if (tok < nvalid) {
+    if (full || tok < nvalid) {
       const float nej = -__expf(bf16_to_f32(pre.w[i]));
       const float dl = ((resets >> tok) & 1u) ? 0.f : cy[i] - pre.e2[i];
       *reinterpret_cast<uint16_t*>(cu.gk + lo * 2 + i * cu.tok_bytes) = f32_to_bf16(dk[i]);
       *reinterpret_cast<uint16_t*>(cu.gb + lo * 2 + i * cu.tok_bytes) = f32_to_bf16(db[i]);
       *reinterpret_cast<uint16_t*>(cu.gw + lo * 2 + i * cu.tok_bytes) = f32_to_bf16(dl * nej);
     }
+  };
+  if (nvalid == CK) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) put(i, true);
+  } else {
+    rare_path();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) put(i, false);
   }
 }
 
