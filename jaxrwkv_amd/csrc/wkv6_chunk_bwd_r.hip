@@ -270,7 +270,7 @@ struct Consumer {
 
 struct Pre {           // per-token scalars at (token 4g+i, key 16q+n), fetched one chunk ahead
   float er[4];
-  uint16_t k[4];
+  uint16_t k[4];   // bf16 bits, widened where they are used: nothing waits for the loads before that
 };
 
 struct Cursor {
@@ -284,13 +284,14 @@ __device__ __forceinline__ void prefetch(Pre& p, const Cursor& cu, int nvalid, i
   const size_t lo = (size_t)cu.voff;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    if (4 * g + i < nvalid) {
-      p.er[i] = *reinterpret_cast<const float*>(cu.er + lo * 4 + 2 * i * cu.tok_bytes);
-      p.k[i] = *reinterpret_cast<const uint16_t*>(cu.k + lo * 2 + i * cu.tok_bytes);
-    } else {
-      p.er[i] = 0.f;
-      p.k[i] = 0;
+    float er = 0.f;
+    uint16_t k = 0;
+    if (nvalid == CK || 4 * g + i < nvalid) {      // the first test is uniform: no lane predicate but in a partial chunk
+      er = *reinterpret_cast<const float*>(cu.er + lo * 4 + 2 * i * cu.tok_bytes);
+      k = *reinterpret_cast<const uint16_t*>(cu.k + lo * 2 + i * cu.tok_bytes);
     }
+    p.er[i] = er;
+    p.k[i] = k;
   }
 }
 

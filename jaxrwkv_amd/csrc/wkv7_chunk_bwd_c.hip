@@ -301,7 +301,7 @@ struct Consumer {
 // fetched one chunk ahead.
 struct Pre {
   float e2[4], e3[4];
-  uint16_t k[4], b[4], w[4];
+  uint16_t k[4], b[4], w[4];   // bf16 bits, widened where they are used: nothing waits for the loads before that
 };
 
 struct Cursor {
@@ -314,27 +314,19 @@ struct Cursor {
 
 __device__ __forceinline__ void prefetch(Pre& p, const Cursor& cu, int nvalid, int g) {
   const size_t lo = (size_t)cu.voff;
-  auto get = [&](int i) {
-    p.e2[i] = *reinterpret_cast<const float*>(cu.e2 + lo * 4 + 2 * i * cu.tok_bytes);
-    p.e3[i] = *reinterpret_cast<const float*>(cu.e3 + lo * 4 + 2 * i * cu.tok_bytes);
-    p.k[i] = *reinterpret_cast<const uint16_t*>(cu.k + lo * 2 + i * cu.tok_bytes);
-    p.b[i] = *reinterpret_cast<const uint16_t*>(cu.b + lo * 2 + i * cu.tok_bytes);
-    p.w[i] = *reinterpret_cast<const uint16_t*>(cu.w + lo * 2 + i * cu.tok_bytes);
-  };
-  if (nvalid == CK) {      // every chunk but a partial last one: no per-lane predicates
 #pragma unroll
-    for (int i = 0; i < 4; ++i) get(i);
-  } else {
-    rare_path();
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      if (4 * g + i < nvalid) {
-        get(i);
-      } else {
-        p.e2[i] = p.e3[i] = 0.f;
-        p.k[i] = p.b[i] = p.w[i] = 0;
-      }
+  for (int i = 0; i < 4; ++i) {
+    float e2 = 0.f, e3 = 0.f;
+    uint16_t k = 0, b = 0, w = 0;
+    if (nvalid == CK || 4 * g + i < nvalid) {      // the first test is uniform: no lane predicate but in a partial chunk
+      e2 = *reinterpret_cast<const float*>(cu.e2 + lo * 4 + 2 * i * cu.tok_bytes);
+      e3 = *reinterpret_cast<const float*>(cu.e3 + lo * 4 + 2 * i * cu.tok_bytes);
+      k = *reinterpret_cast<const uint16_t*>(cu.k + lo * 2 + i * cu.tok_bytes);
+      b = *reinterpret_cast<const uint16_t*>(cu.b + lo * 2 + i * cu.tok_bytes);
+      w = *reinterpret_cast<const uint16_t*>(cu.w + lo * 2 + i * cu.tok_bytes);
     }
+    p.e2[i] = e2; p.e3[i] = e3;
+    p.k[i] = k; p.b[i] = b; p.w[i] = w;
   }
 }
 
