@@ -28,6 +28,7 @@ B, T, H, N = 8, 4096, 32, 64
 # HBM bytes per forward launch of the headline workload, from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`
 # (scaled by a 1 GiB copy; the summary with the commands is profiles/wkv7_fwd_bwd_B8_T4096_H32_bf16.md)
 WKV7_FWD_TRAFFIC_BYTES = 948.5e6
+WKV4_FWD_TRAFFIC_BYTES = 4029.6e6     # profiles/wkv4_fwd_B32_T4096_C2560_f32.md
 
 
 def make_inputs(torch, seed=0):
@@ -113,6 +114,28 @@ def base_record(metric, value, ms_step, args, dtype, workload, extra_config=None
     return {"metric": metric, "value": value, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
             "warmup": args.warmup, "ms_per_step": ms_step, "higher_is_better": True, "scaling": "weak",
             "vs_baseline": None, "dtype": dtype, "data": "synthetic", "config": cfg}
+
+
+def stream_probe(torch):
+    """What a plain streaming kernel reaches on this GPU: torch's c = a + b over three 1 GiB fp32 arrays (two reads
+    and one write per element), bytes moved / HIP-event time.  Reported beside the roofline as the practical
+    ceiling of the memory system; `roofline.peak` stays the published 8 TB/s."""
+    n = (1 << 30) // 4
+    a = torch.ones(n, dtype=torch.float32, device="cuda")
+    b = torch.ones(n, dtype=torch.float32, device="cuda")
+    c = torch.empty(n, dtype=torch.float32, device="cuda")
+    for _ in range(3):
+        torch.add(a, b, out=c)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(10):
+        torch.add(a, b, out=c)
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1) / 10
+    del a, b, c
+    torch.cuda.empty_cache()
+    return {"GB/s": 3 * (1 << 30) / (ms * 1e-3) / 1e9, "pattern": "c = a + b, 1 GiB fp32 each (2 reads + 1 write)"}
 
 
 def roofline(bytes_per_launch, kern_ms, traffic):
@@ -211,7 +234,7 @@ def bench_wkv4(torch, ops, args):
     out = base_record("WKV4 fwd tokens/s (B32 T4096 C2560 fp32)", tokens / (ms_step * 1e-3), ms_step, args, "f32",
                       "isolated WKV4 op, B=32 T=4096 C=2560 fp32, state (0,0,-1e38), length~U{1024..4096} "
                       "(BASELINE configs[3])", {"kernel": "one thread per (sequence, channel)"})
-    out["roofline"] = roofline(fwd_bytes, kern_ms, None)
+    out["roofline"] = roofline(fwd_bytes, kern_ms, WKV4_FWD_TRAFFIC_BYTES)
     return out
 
 
@@ -301,6 +324,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-bwd", action="store_true")
     ap.add_argument("--seq", action="store_true", help="WKV7: force the sequential fp32 VALU kernel")
+    ap.add_argument("--no-stream-probe", action="store_true",
+                    help="skip the streaming-bandwidth probe (three 1 GiB arrays) that is reported beside the roofline")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run three 1 GiB device copies before the timed region (scale for rocprofv3 --pmc)")
     args = ap.parse_args()
@@ -322,6 +347,8 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     out = {"wkv7": bench_wkv7, "wkv6": bench_wkv6, "wkv4": bench_wkv4, "model7": bench_model7}[args.workload](torch, ops, args)
+    if not args.no_stream_probe:
+        out["roofline"]["stream_probe"] = stream_probe(torch)
     print(json.dumps(out))
 
 
