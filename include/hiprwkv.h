@@ -112,7 +112,8 @@ int hiprwkv_wkv6_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype,
 /* ---- WKV4 ------------------------------------------------------------------
  * Replaces ffi target "wkv4-fwd-{fp32,bf16}": operands w,time_first,k,v,s,length,new_starts
  * -> new_s, out  (rwkv4.py:320-321).  `w` = -exp(time_decay) (rwkv4.py:312) and `u` are (C,)
- * io_dtype; the receptance is applied by the caller (rwkv4.py:406). */
+ * io_dtype; the receptance is applied by the caller (rwkv4.py:406).  C <= 2^23.  The output is
+ * num * (1/den) with a 1-ulp reciprocal where the reference divides (difference ~1e-7 relative). */
 int hiprwkv_wkv4_fwd(hiprwkv_stream stream, int io_dtype,
                      int64_t B, int64_t T, int64_t C,
                      const void* w, const void* u, const void* k, const void* v, const void* s,

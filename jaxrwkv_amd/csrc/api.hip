@@ -192,6 +192,8 @@ int hiprwkv_wkv4_fwd(hiprwkv_stream stream, int io_dtype, int64_t B, int64_t T, 
   if (!dtype_ok(io_dtype)) return fail(HIPRWKV_EINVAL, "wkv4_fwd: dtype must be HIPRWKV_F32 or HIPRWKV_BF16");
   if (B <= 0 || T <= 0 || C <= 0) return fail(HIPRWKV_EINVAL, "wkv4_fwd: B,T,C must be positive");
   if (B * ((C + 63) / 64) > 0x7fffffffLL) return fail(HIPRWKV_EINVAL, "wkv4_fwd: B*C exceeds the grid limit");
+  // the forward kernel addresses a block of 32 tokens with 32-bit byte offsets from the block's first token
+  if (C > (1LL << 23)) return fail(HIPRWKV_EINVAL, "wkv4_fwd: C exceeds 2^23 channels");
   const void* req[] = {w, u, k, v, s, new_s, out};
   for (const void* p : req)
     if (p == nullptr) return fail(HIPRWKV_EINVAL, "wkv4_fwd: null tensor pointer");
