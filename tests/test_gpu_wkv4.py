@@ -53,6 +53,28 @@ def test_fp32_forward_shapes(B, T, C, seed, compat, default_state):
     state_close(new_s, ref_s)
 
 
+@pytest.mark.parametrize("T,C,p_reset", [(200, 100, 0.0), (333, 64, 0.004), (96, 257, 0.0), (64, 65, 0.01)])
+def test_fp32_blocks_without_resets(T, C, p_reset):
+    """Long runs of tokens with no reset, sequence end or `length` in them: the kernel's check-free blocks, next
+    to blocks that have one; channel counts that leave part of the last wavefront without a channel of its own."""
+    x = wkv4_inputs(2, T, C, seed=11 + T, p_reset=p_reset, default_state=False, min_len=T // 2)
+    ref_s, ref_y = o4.wkv4_ffi(x["w"], x["u"], x["k"], x["v"], x["s"], x["length"], x["new_starts"], compat=True)
+    new_s, y = run_fwd(x, True)
+    assert_close("y", y, ref_y)
+    state_close(new_s, ref_s)
+
+
+def test_fp32_without_new_starts_pointer():
+    from jaxrwkv_amd import ops
+    x = wkv4_inputs(2, 150, 70, seed=21, default_state=True, min_len=150)
+    ref_s, ref_y = o4.wkv4_ffi(x["w"], x["u"], x["k"], x["v"], x["s"], x["length"], x["new_starts"], compat=True)
+    f = torch.float32
+    new_s, y = ops.wkv4_fwd(dev(x["w"], f), dev(x["u"], f), dev(x["k"], f), dev(x["v"], f), dev(x["s"], f), None, None)
+    torch.cuda.synchronize()
+    assert_close("y", host(y), ref_y)
+    state_close(host(new_s), ref_s)
+
+
 def test_large_k_is_stable():
     x = wkv4_inputs(2, 64, 64, seed=5)
     x["k"] = x["k"] * 60.0
