@@ -72,6 +72,17 @@ __device__ __forceinline__ void split2(float x0, float x1, uint32_t& hi, uint32_
   lo = pack_rn(l0, l1);
 }
 
+// The same split for sources that stay live afterwards (accumulator registers): mask and subtract run at the full
+// VALU rate and leave the source alone, where v_dot2c_f32_bf16 (half rate) accumulates in place and would need a
+// register copy first.
+__device__ __forceinline__ void split2_keep(float x0, float x1, uint32_t& hi, uint32_t& lo) {
+  const uint32_t u0 = __float_as_uint(x0), u1 = __float_as_uint(x1);
+  hi = __builtin_amdgcn_perm(u1, u0, 0x07060302u);
+  const float l0 = x0 - __uint_as_float(u0 & 0xffff0000u);
+  const float l1 = x1 - __uint_as_float(u1 & 0xffff0000u);
+  lo = pack_rn(l0, l1);
+}
+
 // First statement of a rarely taken, wave-uniform branch (resets inside a chunk, the partial last chunk, the chunk
 // of token length-1): keeps the compiler from turning the branch into selects that every chunk would execute.
 __device__ __forceinline__ void rare_path() { asm volatile("" ::: "memory"); }

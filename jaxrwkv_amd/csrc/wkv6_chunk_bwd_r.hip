@@ -324,10 +324,10 @@ __device__ __forceinline__ void split_tiles(const f32x4_t (&G)[4], u32x4_t (&Gh)
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     uint32_t hi, lo;
-    split2(G[2 * j][0], G[2 * j][1], hi, lo); Gh[j][0] = hi; Gl[j][0] = lo;
-    split2(G[2 * j][2], G[2 * j][3], hi, lo); Gh[j][1] = hi; Gl[j][1] = lo;
-    split2(G[2 * j + 1][0], G[2 * j + 1][1], hi, lo); Gh[j][2] = hi; Gl[j][2] = lo;
-    split2(G[2 * j + 1][2], G[2 * j + 1][3], hi, lo); Gh[j][3] = hi; Gl[j][3] = lo;
+    split2_keep(G[2 * j][0], G[2 * j][1], hi, lo); Gh[j][0] = hi; Gl[j][0] = lo;
+    split2_keep(G[2 * j][2], G[2 * j][3], hi, lo); Gh[j][1] = hi; Gl[j][1] = lo;
+    split2_keep(G[2 * j + 1][0], G[2 * j + 1][1], hi, lo); Gh[j][2] = hi; Gl[j][2] = lo;
+    split2_keep(G[2 * j + 1][2], G[2 * j + 1][3], hi, lo); Gh[j][3] = hi; Gl[j][3] = lo;
   }
 }
 

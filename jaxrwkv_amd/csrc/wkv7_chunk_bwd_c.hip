@@ -364,10 +364,10 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     uint32_t hi, lo;
-    split2(C.G[2 * j][0], C.G[2 * j][1], hi, lo); Gh[j][0] = hi; Gl[j][0] = lo;
-    split2(C.G[2 * j][2], C.G[2 * j][3], hi, lo); Gh[j][1] = hi; Gl[j][1] = lo;
-    split2(C.G[2 * j + 1][0], C.G[2 * j + 1][1], hi, lo); Gh[j][2] = hi; Gl[j][2] = lo;
-    split2(C.G[2 * j + 1][2], C.G[2 * j + 1][3], hi, lo); Gh[j][3] = hi; Gl[j][3] = lo;
+    split2_keep(C.G[2 * j][0], C.G[2 * j][1], hi, lo); Gh[j][0] = hi; Gl[j][0] = lo;
+    split2_keep(C.G[2 * j][2], C.G[2 * j][3], hi, lo); Gh[j][1] = hi; Gl[j][1] = lo;
+    split2_keep(C.G[2 * j + 1][0], C.G[2 * j + 1][1], hi, lo); Gh[j][2] = hi; Gl[j][2] = lo;
+    split2_keep(C.G[2 * j + 1][2], C.G[2 * j + 1][3], hi, lo); Gh[j][3] = hi; Gl[j][3] = lo;
   }
   f32x4_t DK = zero4, DB = zero4;   // [token 4g+i][key n]
 #pragma unroll
