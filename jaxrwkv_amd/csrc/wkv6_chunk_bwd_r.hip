@@ -333,7 +333,8 @@ __device__ __forceinline__ void split_tiles(const f32x4_t (&G)[4], u32x4_t (&Gh)
 
 __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ slot, const SnapSlot* __restrict__ snapslot,
                                         const Wkv6Args& A, int64_t b, int64_t h, int nvalid, bool is_snap,
-                                        const Pre& pre, const Cursor& cu) {
+                                        const Pre& pre, Pre& pre_next, const Cursor& cu, const Cursor& cu_next,
+                                        bool has_next) {
   const int lane = C.lane, n = lane & 15, g = lane >> 4, q = C.q;
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
   const u32x4_t rq = *reinterpret_cast<const u32x4_t*>(&slot->RQ[q][lane]);   // B operand: rq of tokens 4g.., hi | lo
@@ -456,16 +457,28 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
     }
     C.carry = cin;
   }
+  uint16_t ok[4], ov[4], ow[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int tok = 4 * g + i;
+    ok[i] = f32_to_bf16(slot->RUC[tok][16 * q + n] + gvk[i]);
+    ov[i] = f32_to_bf16(slot->DYR[tok][16 * q + n] + PV[i] + PV2[i]);
+    ow[i] = f32_to_bf16(((resets >> tok) & 1u) ? 0.f : cy[i] - pre.er[i]);
+  }
+  // The next chunk's per-token scalars are requested after the last read of this chunk's (into a second set of
+  // registers: the caller alternates two sets, so nothing is copied) and before this chunk's stores.  Loads and
+  // stores share one in-order counter, a wait for a load also waits for every older store, and the compiler drains
+  // the counter completely whenever both kinds are in flight: in this order everything in flight at the next wait
+  // is a whole chunk old.  The barriers keep the scheduler from moving the loads up or the stores above them.
+  __builtin_amdgcn_sched_barrier(0);
+  if (has_next) prefetch(pre_next, cu_next, CK, g);
+  __builtin_amdgcn_sched_barrier(0);
   const size_t lo = (size_t)cu.voff;
   auto put = [&](int i, bool full) {
-    const int tok = 4 * g + i;
-    const float dk = slot->RUC[tok][16 * q + n] + gvk[i];
-    const float dv = slot->DYR[tok][16 * q + n] + PV[i] + PV2[i];
-    const float dw = ((resets >> tok) & 1u) ? 0.f : cy[i] - pre.er[i];
-    if (full || tok < nvalid) {
-      *reinterpret_cast<uint16_t*>(cu.gk + lo * 2 + i * cu.tok_bytes) = f32_to_bf16(dk);
-      *reinterpret_cast<uint16_t*>(cu.gv + lo * 2 + i * cu.tok_bytes) = f32_to_bf16(dv);
-      *reinterpret_cast<uint16_t*>(cu.gw + lo * 2 + i * cu.tok_bytes) = f32_to_bf16(dw);
+    if (full || 4 * g + i < nvalid) {
+      *reinterpret_cast<uint16_t*>(cu.gk + lo * 2 + i * cu.tok_bytes) = ok[i];
+      *reinterpret_cast<uint16_t*>(cu.gv + lo * 2 + i * cu.tok_bytes) = ov[i];
+      *reinterpret_cast<uint16_t*>(cu.gw + lo * 2 + i * cu.tok_bytes) = ow[i];
     }
   };
   if (nvalid == CK) {      // every chunk but a partial last one: no per-lane predicates
@@ -518,21 +531,22 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv6_chunk_bwd_r_kernel(
     cu.voff = (uint32_t)((4 * g) * (int)A.H * 64 + 16 * wave + n);
     const int csnap = (L >= 1 && inject) ? (int)((L - 1) / CK) : -1;
     const int tail = (A.T % CK == 0) ? CK : (int)(A.T % CK);
-    Pre pre;
-    if (nch > 0) prefetch(pre, cu, tail, g);
-    for (int j = 0; j < nch; ++j) {
+    Pre pre_a, pre_b;
+    if (nch > 0) prefetch(pre_a, cu, tail, g);
+    auto step = [&](int j, const Pre& pre, Pre& pre_next) {
       const int c = nch - 1 - j;
       const int nvalid = (j == 0) ? tail : CK;
       const int si = j % RING;
-      const Cursor here = cu;
-      const Pre cur = pre;
-      if (j + 1 < nch) {
-        step_back(cu);
-        prefetch(pre, cu, CK, g);
-      }
+      Cursor nxt = cu;
+      step_back(nxt);
       wait_ready(sy, si, j + 1);
-      consume(C, &slots[si], snapslot, A, b, h, nvalid, c == csnap, cur, here);
+      consume(C, &slots[si], snapslot, A, b, h, nvalid, c == csnap, pre, pre_next, cu, nxt, j + 1 < nch);
+      cu = nxt;
       if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    };
+    for (int j = 0; j < nch; j += 2) {      // two steps per turn: the prefetch registers alternate
+      step(j, pre_a, pre_b);
+      if (j + 1 < nch) step(j + 1, pre_b, pre_a);
     }
     // cotangent of the input state; with length == 0 the returned state is the input state itself
     const bool pass = L == 0 && inject;
