@@ -167,10 +167,14 @@ constexpr int W4_SEG = 16;
 
 template <typename IO>
 __global__ __launch_bounds__(W4_THREADS) void wkv4_ckpt_kernel(Wkv4Args A) {
+  static_assert(W4_SEG <= W4_THREADS, "one lane per reset flag of a segment");
   const int64_t cblocks = (A.C + W4_THREADS - 1) / W4_THREADS;
   const int64_t b = blockIdx.x / cblocks;
-  const int64_t c = (blockIdx.x % cblocks) * W4_THREADS + threadIdx.x;
-  if (c >= A.C) return;
+  const int64_t c0 = (blockIdx.x % cblocks) * W4_THREADS + threadIdx.x;
+  // lanes beyond C redo channel C-1 (same loads, same stores of the same values): every lane stays active for the
+  // ballot that gathers a segment's reset flags
+  const int64_t c = c0 < A.C ? c0 : A.C - 1;
+  const int lane = threadIdx.x;
   const IO* kp = reinterpret_cast<const IO*>(A.k) + (size_t)b * A.T * A.C + c;
   const IO* vp = reinterpret_cast<const IO*>(A.v) + (size_t)b * A.T * A.C + c;
   const IO* sp = reinterpret_cast<const IO*>(A.s) + (size_t)b * 3 * A.C + c;
@@ -190,11 +194,15 @@ __global__ __launch_bounds__(W4_THREADS) void wkv4_ckpt_kernel(Wkv4Args A) {
       kc[x] = t < A.T ? ld_f(kp + (size_t)t * A.C) : 0.f;
       vc[x] = t < A.T ? ld_f(vp + (size_t)t * A.C) : 0.f;
     }
+    // one flag per lane, gathered into a uniform mask
+    bool mine = false;
+    if (ns != nullptr && lane < W4_SEG && sg * W4_SEG + lane < A.T) mine = ns[sg * W4_SEG + lane] != 0;
+    const uint32_t rmask = (uint32_t)__ballot(mine);
 #pragma unroll
     for (int x = 0; x < W4_SEG; ++x) {
       const int64_t t = sg * W4_SEG + x;
       if (t < A.T) {
-        if (ns != nullptr && ns[t]) { aa = 0.f; bb = 0.f; pp = W4_RESET_PP; }
+        if ((rmask >> x) & 1u) { aa = 0.f; bb = 0.f; pp = W4_RESET_PP; }
         const float ww = pp + w, diff = ww - kc[x];
         const float e = __expf(-fabsf(diff));
         const float e1 = diff >= 0.f ? 1.f : e, e2 = diff >= 0.f ? e : 1.f;
@@ -210,8 +218,11 @@ template <typename IO>
 __global__ __launch_bounds__(W4_THREADS) void wkv4_bwd_kernel(Wkv4Args A) {
   const int64_t cblocks = (A.C + W4_THREADS - 1) / W4_THREADS;
   const int64_t b = blockIdx.x / cblocks;
-  const int64_t c = (blockIdx.x % cblocks) * W4_THREADS + threadIdx.x;
-  if (c >= A.C) return;
+  const int64_t c0 = (blockIdx.x % cblocks) * W4_THREADS + threadIdx.x;
+  // lanes beyond C redo channel C-1 (same loads, same stores of the same values): every lane stays active for the
+  // ballot that gathers a segment's reset flags
+  const int64_t c = c0 < A.C ? c0 : A.C - 1;
+  const int lane = threadIdx.x;
   const size_t tok0 = (size_t)b * A.T * A.C + c;
   const IO* kp = reinterpret_cast<const IO*>(A.k) + tok0;
   const IO* vp = reinterpret_cast<const IO*>(A.v) + tok0;
@@ -235,7 +246,6 @@ __global__ __launch_bounds__(W4_THREADS) void wkv4_bwd_kernel(Wkv4Args A) {
   for (int64_t sg = nseg - 1; sg >= 0; --sg) {
     const int64_t t0 = sg * W4_SEG;
     float kc[W4_SEG], vc[W4_SEG], gc[W4_SEG], sa[W4_SEG], sb[W4_SEG], spp[W4_SEG];
-    uint32_t rmask = 0;
 #pragma unroll
     for (int x = 0; x < W4_SEG; ++x) {
       const int64_t t = t0 + x;
@@ -243,8 +253,11 @@ __global__ __launch_bounds__(W4_THREADS) void wkv4_bwd_kernel(Wkv4Args A) {
       kc[x] = in ? ld_f(kp + (size_t)t * A.C) : 0.f;
       vc[x] = in ? ld_f(vp + (size_t)t * A.C) : 0.f;
       gc[x] = in ? ld_f(gyp + (size_t)t * A.C) : 0.f;
-      if (in && ns != nullptr && ns[t]) rmask |= 1u << x;
     }
+    // one flag per lane, gathered into a uniform mask
+    bool mine = false;
+    if (ns != nullptr && lane < W4_SEG && t0 + lane < A.T) mine = ns[t0 + lane] != 0;
+    const uint32_t rmask = (uint32_t)__ballot(mine);
     float aa = ck[(sg * 3 + 0) * A.C], bb = ck[(sg * 3 + 1) * A.C], pp = ck[(sg * 3 + 2) * A.C];
     // states entering each step of the segment
 #pragma unroll
