@@ -45,8 +45,8 @@ extern "C" {
 #define HIPRWKV_COMPAT_ASSOC 1u
 /* Force the sequential fp32 VALU kernel even where a chunked MFMA kernel exists. */
 #define HIPRWKV_FORCE_SEQ 2u
-/* hiprwkv_wkv7_fwd runs sequences of at most HIPRWKV_SMALL_T tokens (decode steps) on a kernel that streams the
- * state once and has no per-launch set-up; this flag sends them to the general kernels instead. */
+/* hiprwkv_wkv7_fwd and hiprwkv_wkv6_fwd run sequences of at most HIPRWKV_SMALL_T tokens (decode steps) on a kernel
+ * that streams the state once and has no per-launch set-up; this flag sends them to the general kernels instead. */
 #define HIPRWKV_NO_SMALL_T 4u
 #define HIPRWKV_SMALL_T 8
 

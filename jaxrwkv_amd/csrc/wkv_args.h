@@ -61,6 +61,7 @@ struct Wkv4Args {
 hipError_t launch_wkv7_seq_fwd(const Wkv7Args& A, hipStream_t stream);
 hipError_t launch_wkv7_chunk_fwd(const Wkv7Args& A, hipStream_t stream);
 hipError_t launch_wkv7_small_t_fwd(const Wkv7Args& A, hipStream_t stream);
+hipError_t launch_wkv6_small_t_fwd(const Wkv6Args& A, hipStream_t stream);
 hipError_t launch_wkv7_chunk_bwd_a(const Wkv7Args& A, hipStream_t stream);
 hipError_t launch_wkv7_chunk_bwd_b(const Wkv7Args& A, hipStream_t stream);
 hipError_t launch_wkv7_chunk_bwd_c(const Wkv7Args& A, hipStream_t stream);

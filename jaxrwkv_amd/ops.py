@@ -126,10 +126,11 @@ def wkv7(r, w, k, v, a, b, s, length=None, new_starts=None, compat=True):
 
 
 # ----------------------------------------------------------------------------- WKV6
-def wkv6_fwd(r, k, v, w, u, s, length=None, new_starts=None, compat=True, force_seq=False):
+def wkv6_fwd(r, k, v, w, u, s, length=None, new_starts=None, compat=True, force_seq=False, small_t=True):
     """r,k,v,w (B,T,H,N); u (H,N); s (B,H,N,N) [key, value].  Returns (new_s, y).
 
-    bf16 inputs run on the chunked MFMA kernel unless ``force_seq`` asks for the sequential fp32 one."""
+    T <= 8 runs on the small-T (decode) kernel unless ``small_t=False``; otherwise bf16 inputs run on the chunked
+    MFMA kernel unless ``force_seq`` asks for the sequential fp32 one."""
     lib = _lib.load()
     io = r.dtype
     B, T, H, N = r.shape
@@ -142,7 +143,7 @@ def wkv6_fwd(r, k, v, w, u, s, length=None, new_starts=None, compat=True, force_
     new_s = torch.empty_like(s)
     rc = lib.hiprwkv_wkv6_fwd(_stream(), _DT[io], _DT[s.dtype], B, T, H, N, _p(r), _p(k), _p(v), _p(w), _p(u), _p(s),
                               _p(length), _p(new_starts), _p(y), _p(new_s),
-                              _flags(compat, force_seq))
+                              _flags(compat, force_seq, small_t))
     _lib.check(rc, "hiprwkv_wkv6_fwd")
     return new_s, y
 

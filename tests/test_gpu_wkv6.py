@@ -16,7 +16,8 @@ GOLD = os.path.join(os.path.dirname(__file__), "golden", "wkv6_small.npz")
 def run_fwd(x, dtype, compat):
     from jaxrwkv_amd import ops
     new_s, y = ops.wkv6_fwd(dev(x["r"], dtype), dev(x["k"], dtype), dev(x["v"], dtype), dev(x["w"], dtype),
-                            dev(x["u"], dtype), dev(x["s"]), dev(x["length"]), dev(x["new_starts"]), compat=compat)
+                            dev(x["u"], dtype), dev(x["s"]), dev(x["length"]), dev(x["new_starts"]), compat=compat,
+                            small_t=False)
     torch.cuda.synchronize()
     return host(new_s), host(y)
 

@@ -19,7 +19,7 @@ def run(x, compat, state_dtype=torch.float32, force_seq=False):
     from jaxrwkv_amd import ops
     t = {n: dev(x[n], torch.bfloat16) for n in ("r", "k", "v", "w", "u")}
     new_s, y = ops.wkv6_fwd(t["r"], t["k"], t["v"], t["w"], t["u"], dev(x["s"], state_dtype), dev(x["length"]),
-                            dev(x["new_starts"]), compat=compat, force_seq=force_seq)
+                            dev(x["new_starts"]), compat=compat, force_seq=force_seq, small_t=False)
     torch.cuda.synchronize()
     return host(new_s), host(y)
 
