@@ -44,6 +44,17 @@ __device__ __forceinline__ void st8(bf16_t* p, const float (&o)[8]) {
   *reinterpret_cast<uint4*>(p) = make_uint4(w[0], w[1], w[2], w[3]);
 }
 
+// 16 consecutive elements starting at element `el` of a typed array -> 16 floats
+template <typename T>
+__device__ __forceinline__ void ld16(const void* base, size_t el, float (&o)[16]) {
+  const T* p = reinterpret_cast<const T*>(base) + el;
+  float lo[8], hi[8];
+  ld8(p, lo);
+  ld8(p + 8, hi);
+#pragma unroll
+  for (int c = 0; c < 8; ++c) { o[c] = lo[c]; o[8 + c] = hi[c]; }
+}
+
 // sum over the 4 lanes of a quad (lanes 4m..4m+3); every lane gets the total
 __device__ __forceinline__ float quad_sum(float x) {
   x += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(x), 0xB1, 0xf, 0xf, true));  // quad_perm [1,0,3,2]

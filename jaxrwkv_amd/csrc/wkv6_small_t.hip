@@ -18,16 +18,6 @@ namespace hiprwkv {
 
 namespace {
 
-template <typename T>
-__device__ __forceinline__ void ld16(const void* base, size_t el, float (&o)[16]) {
-  const T* p = reinterpret_cast<const T*>(base) + el;
-  float lo[8], hi[8];
-  ld8(p, lo);
-  ld8(p + 8, hi);
-#pragma unroll
-  for (int c = 0; c < 8; ++c) { o[c] = lo[c]; o[8 + c] = hi[c]; }
-}
-
 template <typename ST>
 __device__ __forceinline__ void st_col(void* base, size_t el, const float (&S)[16], bool zero) {
   ST* p = reinterpret_cast<ST*>(base) + el;
