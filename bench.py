@@ -29,6 +29,7 @@ B, T, H, N = 8, 4096, 32, 64
 # (scaled by a 1 GiB copy; the summary with the commands is profiles/wkv7_fwd_bwd_B8_T4096_H32_bf16.md)
 WKV7_FWD_TRAFFIC_BYTES = 948.5e6
 WKV4_FWD_TRAFFIC_BYTES = 4029.6e6     # profiles/wkv4_fwd_B32_T4096_C2560_f32.md
+WKV6_FWD_TRAFFIC_BYTES = 709.8e6      # profiles/wkv6_fwd_bwd_B16_T2048_H32_bf16.md
 
 
 def make_inputs(torch, seed=0):
@@ -228,7 +229,7 @@ def bench_wkv6(torch, ops, args):
                       "isolated WKV6 op, B=16 T=2048 H=32 N=64 bf16, zero state, new_starts~Bernoulli(1/512) "
                       "(BASELINE configs[2])",
                       {"kernel": "chunked MFMA forward and backward (bf16 hi+lo operands, fp32 accumulate)"})
-    out["roofline"] = roofline(fwd_bytes, kern_ms, None)
+    out["roofline"] = roofline(fwd_bytes, kern_ms, WKV6_FWD_TRAFFIC_BYTES)
     if not args.no_bwd:
         fb = lambda: ops.wkv6_bwd(r, k, v, w, u, s, None, ns, dy, None, compat=True)
         n2 = max(2, args.steps // 4)
