@@ -125,7 +125,7 @@ size_t hiprwkv_wkv4_bwd_workspace_bytes(int64_t B, int64_t T, int64_t C);
 /* Replaces ffi target "wkv4-bwd-{fp32,bf16}": operands w,u,k,v,gy,s,length,new_starts,gs_new
  * -> gw (B,C), gu (B,C), gk, gv, gs  (rwkv4.py:347-349); gw and gu are per sequence in fp32 and are summed
  * over B by the caller (rwkv4.py:351).  gy is the cotangent of the un-gated output.  Unlike the reference's
- * native op it honours gs_new (may be NULL = 0), returns gs, and cuts the chain at new_starts. */
+ * native op it honours gs_new (may be NULL = 0), returns gs, and cuts the chain at new_starts.  C <= 2^23. */
 int hiprwkv_wkv4_bwd(hiprwkv_stream stream, int io_dtype,
                      int64_t B, int64_t T, int64_t C,
                      const void* w, const void* u, const void* k, const void* v, const void* gy, const void* s,

@@ -222,6 +222,7 @@ int hiprwkv_wkv4_bwd(hiprwkv_stream stream, int io_dtype, int64_t B, int64_t T, 
   if (!dtype_ok(io_dtype)) return fail(HIPRWKV_EINVAL, "wkv4_bwd: dtype must be HIPRWKV_F32 or HIPRWKV_BF16");
   if (B <= 0 || T <= 0 || C <= 0) return fail(HIPRWKV_EINVAL, "wkv4_bwd: B,T,C must be positive");
   if (B * ((C + 63) / 64) > 0x7fffffffLL) return fail(HIPRWKV_EINVAL, "wkv4_bwd: B*C exceeds the grid limit");
+  if (C > (1LL << 23)) return fail(HIPRWKV_EINVAL, "wkv4_bwd: C exceeds 2^23 channels");
   const void* req[] = {w, u, k, v, gy, s, gw, gu, gk, gv, gs, workspace};
   for (const void* p : req)
     if (p == nullptr) return fail(HIPRWKV_EINVAL, "wkv4_bwd: null tensor pointer");
