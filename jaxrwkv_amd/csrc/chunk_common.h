@@ -144,17 +144,31 @@ struct ChunkFlags {
 // number of resets at or before in-chunk token t: the index of its segment
 __device__ __forceinline__ int seg_of(uint32_t ns, int t) { return __builtin_popcount(ns & ((2u << t) - 1u)); }
 
-__device__ __forceinline__ ChunkFlags chunk_flags(const uint8_t* ns, unsigned flags, int64_t T, int64_t b, int64_t c0,
-                                                  int64_t L, int lane) {
+// Lanes 0..16 fetch one flag each.  The load has no predicate (lanes beyond the chunk or the sequence re-read the
+// last flag they may, and without flags every lane reads a byte of `dummy`) and its result stays in a register
+// untested, so that a caller can request it a chunk ahead; chunk_flags_of drops what does not belong to the chunk
+// and makes the 17-bit mask uniform with a ballot.
+__device__ __forceinline__ uint32_t chunk_flag_fetch(const uint8_t* ns, const void* dummy, int64_t T, int64_t b,
+                                                     int64_t c0, int lane) {
+  const int64_t room = T - 1 - c0 < CK ? T - 1 - c0 : CK;          // c0 <= T - 1
+  const void* base = ns != nullptr ? static_cast<const void*>(ns + (size_t)b * T + c0) : dummy;
+  const int off = ns != nullptr ? (lane < (int)room ? lane : (int)room) : 0;
+  return __builtin_amdgcn_raw_buffer_load_b8(
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7fffffff, 0x00020000), off, 0, 0);
+}
+__device__ __forceinline__ ChunkFlags chunk_flags_of(const uint8_t* ns, uint32_t mine, unsigned flags, int64_t T,
+                                                     int64_t c0, int64_t L) {
   ChunkFlags F;
   F.compat = (flags & 1u) != 0;
   F.nvalid = (int)((T - c0 < CK) ? (T - c0) : CK);
   F.snap = (L >= 1 && L - 1 >= c0 && L - 1 < c0 + CK) ? (int)(L - 1 - c0) : -1;
-  // lanes 0..16 fetch one flag each; the ballot makes the 17-bit mask uniform
-  bool mine = false;
-  if (ns != nullptr && lane <= CK && c0 + lane < T) mine = ns[(size_t)b * T + c0 + lane] != 0;
-  F.ns = (uint32_t)(__ballot(mine) & 0x1ffffull);
+  const int have = (int)(T - c0 < CK + 1 ? T - c0 : CK + 1);       // flags c0 .. c0 + have - 1 exist
+  F.ns = ns != nullptr ? (uint32_t)(__ballot(mine != 0) & ((1ull << have) - 1ull)) : 0u;
   return F;
+}
+__device__ __forceinline__ ChunkFlags chunk_flags(const uint8_t* ns, unsigned flags, int64_t T, int64_t b, int64_t c0,
+                                                  int64_t L, int lane) {
+  return chunk_flags_of(ns, chunk_flag_fetch(ns, ns, T, b, c0, lane), flags, T, c0, L);
 }
 
 // Selection operands that turn an MFMA into a transposer: against an A operand whose k-slot (g, jj) stands for key
