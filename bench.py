@@ -29,7 +29,7 @@ B, T, H, N = 8, 4096, 32, 64
 # (scaled by a 1 GiB copy; the summary with the commands is profiles/wkv7_fwd_bwd_B8_T4096_H32_bf16.md)
 WKV7_FWD_TRAFFIC_BYTES = 948.5e6
 WKV4_FWD_TRAFFIC_BYTES = 4028.7e6     # profiles/wkv4_fwd_B32_T4096_C2560_f32.md
-WKV6_FWD_TRAFFIC_BYTES = 709.8e6      # profiles/wkv6_fwd_bwd_B16_T2048_H32_bf16.md
+WKV6_FWD_TRAFFIC_BYTES = 701.6e6      # profiles/wkv6_fwd_bwd_B16_T2048_H32_bf16.md
 
 
 def make_inputs(torch, seed=0):
