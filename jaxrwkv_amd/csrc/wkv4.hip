@@ -70,6 +70,17 @@ __device__ __forceinline__ void buf_st(bf16_t*, float x, rsrc_t r, int voff, int
   __builtin_amdgcn_raw_buffer_store_b16(f32_to_bf16(x), r, voff, soff, 0);
 }
 
+// this lane's reset flag of the run of tokens that starts at token tb (lane x: token tb + x, clamped into the
+// sequence: lanes beyond it re-read its last flag and are masked by the caller); without flags every lane reads a
+// byte of `dummy` that is then ignored
+__device__ __forceinline__ uint32_t seg_flag(const uint8_t* ns, const void* dummy, int64_t tb, int64_t T, int lane) {
+  const int64_t fb = tb < T - 1 ? tb : T - 1;
+  const int room = (int)(T - 1 - fb < 63 ? T - 1 - fb : 63);
+  const void* base = ns != nullptr ? static_cast<const void*>(ns + fb) : dummy;
+  const int off = ns != nullptr ? (lane < room ? lane : room) : 0;
+  return __builtin_amdgcn_raw_buffer_load_b8(make_rsrc(base), off, 0, 0);
+}
+
 }  // namespace
 
 template <typename IO>
@@ -111,13 +122,7 @@ __global__ __launch_bounds__(W4_THREADS) void wkv4_fwd_kernel(Wkv4Args A) {
   // re-read row T-1 and are never used, so no request needs a predicate.
   float kr[W4_TB], vr[W4_TB];
   uint32_t nsb;                                      // this lane's reset flag of the block after the current one
-  // flags of the block starting at token tb (lane x: token tb + x, clamped into the sequence)
-  auto fetch_flags = [&](int64_t tb) {
-    const int64_t fb = tb < A.T - 1 ? tb : A.T - 1;
-    const int room = (int)(A.T - 1 - fb < 63 ? A.T - 1 - fb : 63);
-    const void* base = ns != nullptr ? static_cast<const void*>(ns + fb) : static_cast<const void*>(kseq);
-    nsb = __builtin_amdgcn_raw_buffer_load_b8(make_rsrc(base), ns != nullptr && lane < room ? lane : (ns != nullptr ? room : 0), 0, 0);
-  };
+  auto fetch_flags = [&](int64_t tb) { nsb = seg_flag(ns, kseq, tb, A.T, lane); };
   fetch_flags(0);
   {
     const rsrc_t rk = make_rsrc(kseq), rv = make_rsrc(vseq);
@@ -181,15 +186,6 @@ constexpr int W4_SEG = 16;
 
 namespace {
 
-// this lane's reset flag of the segment that starts at token tb (lane x: token tb + x, clamped into the sequence);
-// without flags every lane reads a byte of `dummy` that is then ignored
-__device__ __forceinline__ uint32_t seg_flag(const uint8_t* ns, const void* dummy, int64_t tb, int64_t T, int lane) {
-  const int64_t fb = tb < T - 1 ? tb : T - 1;
-  const int room = (int)(T - 1 - fb < 63 ? T - 1 - fb : 63);
-  const void* base = ns != nullptr ? static_cast<const void*>(ns + fb) : dummy;
-  const int off = ns != nullptr ? (lane < room ? lane : room) : 0;
-  return __builtin_amdgcn_raw_buffer_load_b8(make_rsrc(base), off, 0, 0);
-}
 // the flags of a segment as a uniform mask, bit x = token t0 + x (tokens beyond the sequence have none)
 __device__ __forceinline__ uint32_t seg_mask(const uint8_t* ns, uint32_t flag, int64_t t0, int64_t T) {
   if (ns == nullptr) return 0u;
