@@ -1,5 +1,6 @@
-// WKV7 backward, forward sweep B on the matrix cores (bf16 I/O, gfx950): gr, ga and the two per-token workspaces
-// e2 = a.da, e3 = r.dr (+ <dS_out, S> at token length-1) that the decay-gradient recursion of sweep C consumes.
+// WKV7 backward, forward sweep B on the matrix cores (bf16 I/O, gfx950): gr, ga and the per-token workspace
+// f_t = e3_t + e2_{t+1} (e2 = a.da, dropped when token t+1 starts a sequence; e3 = r.dr + <dS_out, S> at token
+// length-1) that the decay-gradient recursion of sweep C consumes.
 //
 // With sa_t known from the forward pass the state obeys a linear recurrence (S[i][j] = value row i, key col j):
 //     S_t = S_{t-1} diag(d_t) + sa_t b_t^T + v_t k_t^T ;   dr_t = S_t^T dy_t ;   da_t = S_{t-1}^T dsa_t
@@ -51,7 +52,7 @@ struct __attribute__((aligned(16))) Slot {
   int snap;                    // -1, or the in-chunk index of token length-1
   int keep_end;                // the entering state survives to the chunk end (no reset in the chunk)
   int keep_snap;               // the entering state survives to token length-1
-  int pad;
+  int ns;                      // bit t: new_starts of in-chunk token t; bit 16: of the first token of the next chunk
 };
 struct __attribute__((aligned(16))) SnapSlot {
   uint4 SAt[4][64];            // update operands with the tokens masked for the state at token length-1
@@ -286,6 +287,7 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
     slot->snap = F.snap;
     slot->keep_end = (lastseg == 0) ? 1 : 0;
     slot->keep_snap = (F.snap >= 0 && (!slow || seg_of(F.ns, F.snap) == 0)) ? 1 : 0;
+    slot->ns = (int)F.ns;
   }
 }
 
@@ -294,12 +296,13 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
 // g = lane/16), S[vt][i] = S[value 16*vt + 4g + i][key 16q + n].
 struct Consumer {
   f32x4_t S[4];
+  float pend;          // lanes g = 3: r.dr of the previous chunk's last token, whose workspace entry is still open
   int q, lane;
 };
 
 struct OutCursor {
   char *gr, *ga;       // bf16 outputs at (b, c0, h, 0)
-  char *e2, *e3;       // fp32 workspaces at the same place
+  char* ef;            // fp32 workspace at the same place
   size_t tok_bytes;    // bytes between consecutive tokens in the bf16 arrays (twice that in the fp32 ones)
   uint32_t voff;       // lane part of the address, in elements: (4g * H) * 64 + key
 };
@@ -312,7 +315,8 @@ __device__ __forceinline__ float ld_state_el(const void* p, int f32, size_t off)
 }
 
 __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ slot, const SnapSlot* __restrict__ snapslot,
-                                        const Wkv7Args& A, int64_t b, int64_t h, int nvalid, bool is_snap, OutCursor& oc) {
+                                        const Wkv7Args& A, int64_t b, int64_t h, int nvalid, bool is_snap, bool first,
+                                        bool last, OutCursor& oc) {
   const int lane = C.lane, n = lane & 15, g = lane >> 4, q = C.q;
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
   // B operands of the token contractions: (b/E, k/E) of tokens 4g..4g+3 at this wave's keys
@@ -403,29 +407,51 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
 #pragma unroll
   for (int i = 0; i < 5; ++i) e[i] = slot->E[4 * g + i][16 * q + n];
   const size_t lo = (size_t)oc.voff;
-  auto put = [&](int i, bool full) {
+  const bool full = nvalid == CK;      // every chunk but a partial last one: no per-lane predicates
+  float e2[4], e3[4];
+  uint16_t odr[4], oda[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
     const int tok = 4 * g + i;
     const float rr = bf16_to_f32(slot->RA[0][tok][16 * q + n]);
     const float aa = bf16_to_f32(slot->RA[1][tok][16 * q + n]);
     const float dr = DR[i] * e[i + 1];
     const float da = DA[i] * e[i];
-    if (full || tok < nvalid) {
-      *reinterpret_cast<uint16_t*>(oc.gr + lo * 2 + i * oc.tok_bytes) = f32_to_bf16(dr);
-      *reinterpret_cast<uint16_t*>(oc.ga + lo * 2 + i * oc.tok_bytes) = f32_to_bf16(da);
-      *reinterpret_cast<float*>(oc.e2 + lo * 4 + 2 * i * oc.tok_bytes) = aa * da;
-      *reinterpret_cast<float*>(oc.e3 + lo * 4 + 2 * i * oc.tok_bytes) = fmaf(rr, dr, tok == snap_tok ? inj : 0.f);
-    }
-  };
-  if (nvalid == CK) {      // every chunk but a partial last one: no per-lane predicates
-#pragma unroll
-    for (int i = 0; i < 4; ++i) put(i, true);
-  } else {
+    odr[i] = f32_to_bf16(dr); oda[i] = f32_to_bf16(da);
+    e2[i] = aa * da;
+    e3[i] = fmaf(rr, dr, tok == snap_tok ? inj : 0.f);
+  }
+  if (!full) {
     rare_path();
 #pragma unroll
-    for (int i = 0; i < 4; ++i) put(i, false);
+    for (int i = 0; i < 4; ++i)
+      if (4 * g + i >= nvalid) e2[i] = 0.f;          // nothing follows the last token of the sequence
   }
+  // What the decay-gradient recursion of sweep C adds at token t is e3_t + e2_{t+1}, without e2_{t+1} when token
+  // t+1 starts a sequence.  e2 of the next token lives in this lane, in the lane 16 further on (token 4g+4), or in
+  // the next chunk: the entry of token 15 stays open until then.
+  const uint32_t nsm = (uint32_t)slot->ns;
+  auto follows = [&](int tok) { return ((nsm >> tok) & 1u) == 0; };   // token `tok` continues the sequence of tok-1
+  const float up = __shfl_down(e2[0], 16, 64);
+  float f[4];
+#pragma unroll
+  for (int i = 0; i < 3; ++i) f[i] = e3[i] + (follows(4 * g + i + 1) ? e2[i + 1] : 0.f);
+  f[3] = e3[3] + ((g < 3 && follows(4 * g + 4)) ? up : 0.f);
+  const float open_prev = __shfl(C.pend, n + 48, 64);   // the previous chunk's token 15, handed to the lanes of token 0
+  C.pend = e3[3];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    if (full || 4 * g + i < nvalid) {
+      *reinterpret_cast<uint16_t*>(oc.gr + lo * 2 + i * oc.tok_bytes) = odr[i];
+      *reinterpret_cast<uint16_t*>(oc.ga + lo * 2 + i * oc.tok_bytes) = oda[i];
+      // token 15 of a full chunk that is not the last one waits for the next chunk (below)
+      if (i < 3 || g < 3 || last) *reinterpret_cast<float*>(oc.ef + lo * 4 + 2 * i * oc.tok_bytes) = f[i];
+    }
+  }
+  if (!first && g == 0)
+    *reinterpret_cast<float*>(oc.ef + lo * 4 - 2 * oc.tok_bytes) = open_prev + (follows(0) ? e2[0] : 0.f);
   oc.gr += CK * oc.tok_bytes; oc.ga += CK * oc.tok_bytes;
-  oc.e2 += 2 * CK * oc.tok_bytes; oc.e3 += 2 * CK * oc.tok_bytes;
+  oc.ef += 2 * CK * oc.tok_bytes;
 }
 
 }  // namespace
@@ -454,6 +480,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_bwd_b_kernel(
     Consumer C;
     C.q = wave;
     C.lane = lane;
+    C.pend = 0.f;
     const int n = lane & 15, g = lane >> 4;
 #pragma unroll
     for (int vt = 0; vt < 4; ++vt)
@@ -465,15 +492,14 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_bwd_b_kernel(
     const size_t el0 = (((size_t)b * A.T) * A.H + h) * 64;
     oc.gr = reinterpret_cast<char*>(A.gr) + el0 * 2;
     oc.ga = reinterpret_cast<char*>(A.ga) + el0 * 2;
-    oc.e2 = reinterpret_cast<char*>(A.e2) + el0 * 4;
-    oc.e3 = reinterpret_cast<char*>(A.e3) + el0 * 4;
+    oc.ef = reinterpret_cast<char*>(A.e2) + el0 * 4;
     oc.voff = (uint32_t)((4 * g) * (int)A.H * 64 + 16 * wave + n);
     const int csnap = (L >= 1 && inject) ? (int)((L - 1) / CK) : -1;
     for (int c = 0; c < nch; ++c) {
       const int nvalid = (c + 1 < nch || A.T % CK == 0) ? CK : (int)(A.T % CK);
       const int si = c % RING;
       wait_ready(sy, si, c + 1);
-      consume(C, &slots[si], snapslot, A, b, h, nvalid, c == csnap, oc);
+      consume(C, &slots[si], snapslot, A, b, h, nvalid, c == csnap, c == 0, c + 1 == nch, oc);
       // every LDS read of slot si has returned: its data went into the MFMAs and stores above
       if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], c + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }

@@ -13,7 +13,9 @@
 // Kh <-> Qt) and the decay applied before the update.  The decay gradient needs <G_t, S'_t> per key; as in the
 // sequential sweep it comes from the running sum
 //     carry_t = reset_t ? 0 : carry_{t+1} + e3_t + e2_t - k_t.dk_t - b_t.db_t ;   dw_t = (carry_t - e2_t) * (-exp(w_t))
-// with e2 = a.da and e3 = r.dr (+ <dS_out, S> at token length-1) left by sweep B.
+// with e2 = a.da and e3 = r.dr (+ <dS_out, S> at token length-1).  In terms of c_t = carry_t - e2_t (c_t = 0 at a
+// reset) this is c_t = reset_t ? 0 : c_{t+1} + f_t - k_t.dk_t - b_t.db_t, dw_t = c_t * (-exp(w_t)), with the one
+// vector f_t = e3_t + (reset_{t+1} ? 0 : e2_{t+1}) per token that sweep B leaves.
 //
 // Work split as in sweep B: 4 consumer waves hold G split by key columns (value x key accumulator tiles reused
 // as B operands), 4 producer waves prepare the state-independent operands into a ring of LDS slots; bounded-poll
@@ -300,12 +302,12 @@ struct Consumer {
 // Per-token scalars at (token 4g+i, key 16q+n) that the decay-gradient recursion reads from global memory,
 // fetched one chunk ahead.
 struct Pre {
-  float e2[4], e3[4];
+  float f[4];                  // e3_t + e2_{t+1}, left by sweep B
   uint16_t k[4], b[4], w[4];   // bf16 bits, widened where they are used: nothing waits for the loads before that
 };
 
 struct Cursor {
-  const char *e2, *e3;         // fp32 workspaces at (b, c0, h, 0)
+  const char* ef;              // fp32 workspace at (b, c0, h, 0)
   const char *k, *b, *w;       // bf16 inputs at the same place
   char *gk, *gb, *gw;          // bf16 outputs
   size_t tok_bytes;            // bytes between consecutive tokens in the bf16 arrays (twice that in the fp32 ones)
@@ -316,23 +318,22 @@ __device__ __forceinline__ void prefetch(Pre& p, const Cursor& cu, int nvalid, i
   const size_t lo = (size_t)cu.voff;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    float e2 = 0.f, e3 = 0.f;
+    float f = 0.f;
     uint16_t k = 0, b = 0, w = 0;
     if (nvalid == CK || 4 * g + i < nvalid) {      // the first test is uniform: no lane predicate but in a partial chunk
-      e2 = *reinterpret_cast<const float*>(cu.e2 + lo * 4 + 2 * i * cu.tok_bytes);
-      e3 = *reinterpret_cast<const float*>(cu.e3 + lo * 4 + 2 * i * cu.tok_bytes);
+      f = *reinterpret_cast<const float*>(cu.ef + lo * 4 + 2 * i * cu.tok_bytes);
       k = *reinterpret_cast<const uint16_t*>(cu.k + lo * 2 + i * cu.tok_bytes);
       b = *reinterpret_cast<const uint16_t*>(cu.b + lo * 2 + i * cu.tok_bytes);
       w = *reinterpret_cast<const uint16_t*>(cu.w + lo * 2 + i * cu.tok_bytes);
     }
-    p.e2[i] = e2; p.e3[i] = e3;
+    p.f[i] = f;
     p.k[i] = k; p.b[i] = b; p.w[i] = w;
   }
 }
 
 __device__ __forceinline__ void step_back(Cursor& cu) {
   const size_t d = CK * cu.tok_bytes;
-  cu.e2 -= 2 * d; cu.e3 -= 2 * d;
+  cu.ef -= 2 * d;
   cu.k -= d; cu.b -= d; cu.w -= d;
   cu.gk -= d; cu.gb -= d; cu.gw -= d;
 }
@@ -441,7 +442,7 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
     dk[i] = DK[i] * ei;
     db[i] = DB[i] * ei;
     const float kk = bf16_to_f32(pre.k[i]), bb = bf16_to_f32(pre.b[i]);
-    z[i] = pre.e3[i] + pre.e2[i] - kk * dk[i] - bb * db[i];
+    z[i] = pre.f[i] - kk * dk[i] - bb * db[i];
   }
   // carry_t = reset_t ? 0 : carry_{t+1} + z_t, from token 15 down
   if (resets == 0) {
@@ -463,10 +464,8 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
   uint16_t ok[4], ob[4], ow[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int tok = 4 * g + i;
     const float nej = -__expf(bf16_to_f32(pre.w[i]));
-    const float dl = ((resets >> tok) & 1u) ? 0.f : cy[i] - pre.e2[i];
-    ok[i] = f32_to_bf16(dk[i]); ob[i] = f32_to_bf16(db[i]); ow[i] = f32_to_bf16(dl * nej);
+    ok[i] = f32_to_bf16(dk[i]); ob[i] = f32_to_bf16(db[i]); ow[i] = f32_to_bf16(cy[i] * nej);
   }
   // The next chunk's per-token scalars are requested after the last read of this chunk's (into a second set of
   // registers: the caller alternates two sets, so nothing is copied) and before this chunk's stores.  Loads and
@@ -528,8 +527,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_bwd_c_kernel(
     Cursor cu;
     cu.tok_bytes = (size_t)A.H * 64 * 2;
     const size_t el0 = (((size_t)b * A.T + (size_t)(nch - 1) * CK) * A.H + h) * 64;
-    cu.e2 = reinterpret_cast<const char*>(A.e2) + el0 * 4;
-    cu.e3 = reinterpret_cast<const char*>(A.e3) + el0 * 4;
+    cu.ef = reinterpret_cast<const char*>(A.e2) + el0 * 4;
     cu.k = reinterpret_cast<const char*>(A.k) + el0 * 2;
     cu.b = reinterpret_cast<const char*>(A.b) + el0 * 2;
     cu.w = reinterpret_cast<const char*>(A.w) + el0 * 2;
