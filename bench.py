@@ -202,7 +202,7 @@ def bench_wkv7(torch, ops, args):
                           "hbm_frac": fb_bytes / (ms2 * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": fb_bytes,
                           "note": "backward = three sweeps (reverse, forward, reverse), " +
                                   ("sequential fp32 VALU kernels" if args.seq else "chunked MFMA kernels") +
-                                  "; dsa, e2, e3 pass through an fp32 workspace"}
+                                  "; dsa and the decay-gradient terms pass through an fp32 workspace"}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
         out["cpu_baseline_sequential"] = cpu_baseline_sequential()

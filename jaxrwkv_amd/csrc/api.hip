@@ -105,7 +105,8 @@ int hiprwkv_wkv7_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64
   A.dsa = reinterpret_cast<float*>(ws);
   A.e2 = reinterpret_cast<float*>(ws + one);
   A.e3 = reinterpret_cast<float*>(ws + 2 * one);
-  // Three sweeps: A (reverse) -> gv, dsa, gs; B (forward) -> gr, ga, e2, e3; C (reverse) -> gk, gb, gw.
+  // Three sweeps: A (reverse) -> gv, dsa, gs; B (forward) -> gr, ga, e2, e3 (the chunked B: their sum shifted by a
+  // token, in e2); C (reverse) -> gk, gb, gw.
   // bf16 I/O runs all three on the chunked MFMA kernels.
   const bool chunked = io_dtype == HIPRWKV_BF16 && !(flags & HIPRWKV_FORCE_SEQ);
   hipStream_t st = static_cast<hipStream_t>(stream);

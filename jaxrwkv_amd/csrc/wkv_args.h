@@ -20,7 +20,7 @@ struct Wkv7Args {
   const float* sa_in;
   const void* gs_out;
   void *gw, *gr, *gk, *gv, *ga, *gb, *gs;
-  float *dsa, *e2, *e3;  // workspace, (B,T,H,64) fp32 each
+  float *dsa, *e2, *e3;  // workspace, (B,T,H,64) fp32 each (the chunked sweeps keep e3_t + e2_{t+1} in e2, e3 unused)
 };
 
 struct Wkv6Args {
