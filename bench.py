@@ -84,7 +84,7 @@ def time_region(torch, fn, steps, warmup, prewarm_s=PREWARM_S):
     return wall, e0.elapsed_time(e1) / steps
 
 
-def cpu_baseline(sample_heads=2, threads=None, target_s=10.0, max_heads=16):
+def cpu_baseline(sample_heads=2, threads=None, target_s=15.0, max_heads=32):
     """Oracle's AssociativeScanRWKV restatement (log-depth scan, fp32) on the host: one sequence of the benchmark
     shape restricted to a few of the 32 heads; tokens/s is scaled to all heads of a token.  A first pass over
     `sample_heads` heads sizes a second one (at most `max_heads`, for memory) to about `target_s` seconds of work
