@@ -82,7 +82,7 @@ __device__ __forceinline__ void load_raw(Raw& x, const Wkv6Args& A, int64_t b, i
 struct Producer {
   int lane;
   u32x4_t sel[2];     // MFMA-as-transposer selection operands
-  const char* u;      // the bonus of this lane's keys (bf16): 16 bytes here and 16 bytes 64 bytes further on
+  const char* u;      // the bonus of this lane's keys (bf16, staged in LDS): 16 bytes here and 16 bytes 64 bytes on
 };
 
 __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const ChunkFlags& F, Slot* __restrict__ slot,
@@ -154,7 +154,7 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
     {
       float fr[8], fk[8], fu[8], Einv[8], Ee[8];
       unpack8(x.r[hf], fr); unpack8(x.k[hf], fk);
-      unpack8(*reinterpret_cast<const uint4*>(P.u + 64 * hf), fu);   // re-read per chunk (cache hit): frees registers
+      unpack8(*reinterpret_cast<const uint4*>(P.u + 64 * hf), fu);   // re-read per chunk from LDS: frees registers
 #pragma unroll
       for (int e = 0; e < 8; ++e) {
         const float l2 = fmaxf(E[e], MIN_CUM_L2);
@@ -400,6 +400,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD), 4) void wkv6_chunk_fwd_kernel
   Slot* slots = reinterpret_cast<Slot*>(smem_raw);
   SnapSlot* snapslot = reinterpret_cast<SnapSlot*>(smem_raw + RING * sizeof(Slot));
   Sync* sy = reinterpret_cast<Sync*>(smem_raw + RING * sizeof(Slot) + sizeof(SnapSlot));
+  uint16_t* ulds = reinterpret_cast<uint16_t*>(smem_raw + RING * sizeof(Slot) + sizeof(SnapSlot) + sizeof(Sync));   // u of this head
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   const int64_t b = blockIdx.x / A.H, h = blockIdx.x % A.H;
@@ -407,6 +408,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD), 4) void wkv6_chunk_fwd_kernel
   L = L < A.T ? L : A.T;
   const int64_t nchunks = (A.T + CK - 1) / CK;
   if (threadIdx.x < sizeof(Sync) / sizeof(int)) reinterpret_cast<int*>(sy)[threadIdx.x] = 0;
+  if (threadIdx.x < 64) ulds[threadIdx.x] = reinterpret_cast<const uint16_t*>(A.u)[(size_t)(blockIdx.x % A.H) * 64 + threadIdx.x];
   __syncthreads();
 
   if (wave < NCONS) {
@@ -442,7 +444,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD), 4) void wkv6_chunk_fwd_kernel
     Producer P;
     P.lane = lane;
     make_sel(P.sel, lane);
-    P.u = reinterpret_cast<const char*>(A.u) + ((size_t)h * 64 + 8 * (lane >> 4)) * 2;
+    P.u = reinterpret_cast<const char*>(ulds) + 8 * (lane >> 4) * 2;
     Raw raw;
     if (p < nchunks) load_raw(raw, A, b, h, (int64_t)p * CK, lane);
     for (int64_t c = p; c < nchunks; c += NPROD) {
@@ -460,7 +462,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD), 4) void wkv6_chunk_fwd_kernel
 }
 
 hipError_t launch_wkv6_chunk_fwd(const Wkv6Args& A, hipStream_t stream) {
-  const size_t smem = RING * sizeof(Slot) + sizeof(SnapSlot) + sizeof(Sync);
+  const size_t smem = RING * sizeof(Slot) + sizeof(SnapSlot) + sizeof(Sync) + 64 * sizeof(uint16_t);
   hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(wkv6_chunk_fwd_kernel),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
   if (e != hipSuccess) return e;
