@@ -44,6 +44,12 @@ def test_argument_validation_without_gpu():
     assert rc == -1 and b"dtype" in lib.hiprwkv_last_error()
     rc = lib.hiprwkv_wkv4_fwd(null, 0, 0, 8, 64, *([null] * 9), 0)
     assert rc == -1
+    # WKV4 channel limit (32-bit byte offsets inside a block of tokens), forward and backward
+    rc = lib.hiprwkv_wkv4_fwd(null, 0, 1, 8, (1 << 23) + 1, *([null] * 9), 0)
+    assert rc == -1 and b"2^23" in lib.hiprwkv_last_error()
+    rc = lib.hiprwkv_wkv4_bwd(null, 0, 1, 8, (1 << 23) + 1, *([null] * 14), null, 0, 0)
+    assert rc == -1 and b"2^23" in lib.hiprwkv_last_error()
+    assert lib.hiprwkv_wkv4_bwd_workspace_bytes(2, 17, 64) >= 2 * 2 * 3 * 64 * 4
     assert lib.hiprwkv_wkv7_bwd_workspace_bytes(2, 16, 2, 64) == 3 * 2 * 16 * 2 * 64 * 4
     assert lib.hiprwkv_wkv6_bwd_workspace_bytes(2, 16, 2, 64) >= 2 * 16 * 2 * 64 * 4
 
