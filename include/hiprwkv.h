@@ -3,7 +3,7 @@
  *
  * Every entry point only enqueues work on the caller's HIP stream: it does not
  * allocate, free or synchronise, so it can be called from an XLA custom-call
- * handler thread.  All pointers are device pointers.  Entry points return
+ * handler thread.  All pointers are device pointers, 16-byte aligned.  Entry points return
  * HIPRWKV_OK or a negative HIPRWKV_E* code; hiprwkv_last_error() then returns a
  * thread-local message.
  *
@@ -49,11 +49,22 @@ extern "C" {
  * that streams the state once and has no per-launch set-up; this flag sends them to the general kernels instead. */
 #define HIPRWKV_NO_SMALL_T 4u
 #define HIPRWKV_SMALL_T 8
+/* Test hook for the chunked kernels' bounded hand-shake: the producer wave of the last chunk does not publish it, the
+ * consumer waves' wait runs out (a few milliseconds), every wave still ends normally, the outputs of every
+ * (sequence, head) are NaN and hiprwkv_handshake_failures() has advanced by B*H per kernel. */
+#define HIPRWKV_DEBUG_DROP_PUBLISH 0x100u
 
 typedef void* hiprwkv_stream; /* a hipStream_t */
 
 const char* hiprwkv_last_error(void);
 int hiprwkv_version(void);
+
+/* The chunked kernels pass work between waves of a workgroup through a hand-shake with a bounded wait (a broken
+ * hand-shake must not hang the GPU).  A workgroup whose wait runs out overwrites all its outputs for that
+ * (sequence, head) with NaN and adds one to a per-device counter; this call copies the counter of the current
+ * device to *count (host memory).  Unlike every other entry point it synchronises `stream`.  No counterpart in
+ * the reference; for health checks and tests. */
+int hiprwkv_handshake_failures(hiprwkv_stream stream, unsigned* count);
 
 /* ---- WKV7 ------------------------------------------------------------------
  * Replaces ffi target "wkv7-fwd-{fp32,bf16}": operands w,r,k,v,a,b,s,length,new_starts

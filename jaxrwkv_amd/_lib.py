@@ -12,6 +12,7 @@ F32, BF16 = 0, 1
 COMPAT_ASSOC = 1
 FORCE_SEQ = 2
 NO_SMALL_T = 4
+DEBUG_DROP_PUBLISH = 0x100
 
 _vp, _i64, _int, _u32, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_uint, ctypes.c_size_t
 
@@ -19,6 +20,7 @@ _vp, _i64, _int, _u32, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctyp
 SIGNATURES = {
     "hiprwkv_last_error": (ctypes.c_char_p, []),
     "hiprwkv_version": (_int, []),
+    "hiprwkv_handshake_failures": (_int, [_vp, ctypes.POINTER(ctypes.c_uint)]),
     "hiprwkv_wkv7_fwd": (_int, [_vp, _int, _int, _i64, _i64, _i64, _i64] + [_vp] * 7 + [_vp, _vp] + [_vp, _vp, _vp, _u32]),
     "hiprwkv_wkv7_bwd_workspace_bytes": (_sz, [_i64] * 4),
     "hiprwkv_wkv7_bwd": (_int, [_vp, _int, _int, _i64, _i64, _i64, _i64] + [_vp] * 7 + [_vp, _vp] + [_vp] * 3

@@ -5,6 +5,8 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "wkv_args.h"
 
 using namespace hiprwkv;
@@ -35,12 +37,45 @@ int check_matrix_shape(const char* op, int io_dtype, int state_dtype, int64_t B,
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
+// Counts the workgroups of the chunked kernels whose bounded hand-shake wait ran out (they overwrite their outputs
+// with NaN and add one here).  Every GPU holds its own copy of the word; its address is looked up once per device.
+__device__ unsigned int g_handshake_failures = 0u;
+
+constexpr int MAX_DEVICES = 64;
+std::mutex g_sym_mu;
+unsigned* g_status_ptr[MAX_DEVICES] = {};
+
+// Address of the current device's failure counter, or null when it cannot be obtained (the kernels then skip the
+// count; the NaN poisoning does not depend on it).
+unsigned* status_word() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) return nullptr;
+  std::lock_guard<std::mutex> lock(g_sym_mu);
+  if (g_status_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_handshake_failures)) != hipSuccess) return nullptr;
+    g_status_ptr[dev] = static_cast<unsigned*>(p);
+  }
+  return g_status_ptr[dev];
+}
+
 }  // namespace
 
 extern "C" {
 
 const char* hiprwkv_last_error(void) { return g_err; }
-int hiprwkv_version(void) { return 100; }
+int hiprwkv_version(void) { return 101; }
+
+int hiprwkv_handshake_failures(hiprwkv_stream stream, unsigned* count) {
+  if (count == nullptr) return fail(HIPRWKV_EINVAL, "handshake_failures: null count pointer");
+  unsigned* word = status_word();
+  if (word == nullptr) return fail(HIPRWKV_ELAUNCH, "handshake_failures: the device counter is not reachable");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipError_t e = hipMemcpyAsync(count, word, sizeof(unsigned), hipMemcpyDeviceToHost, st);
+  if (e == hipSuccess) e = hipStreamSynchronize(st);
+  if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "handshake_failures: %s", hipGetErrorString(e));
+  return HIPRWKV_OK;
+}
 
 int hiprwkv_wkv7_fwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64_t B, int64_t T, int64_t H, int64_t N,
                      const void* w, const void* r, const void* k, const void* v, const void* a, const void* b,
@@ -62,6 +97,7 @@ int hiprwkv_wkv7_fwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64
   A.out = out; A.sa = sa; A.new_s = new_s;
   A.io_f32 = io_dtype == HIPRWKV_F32; A.st_f32 = state_dtype == HIPRWKV_F32;
   A.flags = flags;
+  A.status = status_word();
   // T <= 8 (decode) runs on the small-T kernel; otherwise bf16 I/O on the chunked MFMA kernel and fp32 I/O (and
   // HIPRWKV_FORCE_SEQ) on the exact sequential one
   const bool small_t = T <= HIPRWKV_SMALL_T && !(flags & HIPRWKV_NO_SMALL_T);
@@ -98,6 +134,7 @@ int hiprwkv_wkv7_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64
   A.length = length; A.ns = new_starts;
   A.io_f32 = io_dtype == HIPRWKV_F32; A.st_f32 = state_dtype == HIPRWKV_F32;
   A.flags = flags;
+  A.status = status_word();
   A.gy = gy; A.sa_in = sa; A.gs_out = gs_out;
   A.gw = gw; A.gr = gr; A.gk = gk; A.gv = gv; A.ga = ga; A.gb = gb; A.gs = gs;
   const size_t one = need / 3;
@@ -135,6 +172,7 @@ int hiprwkv_wkv6_fwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64
   A.out = out; A.new_s = new_s;
   A.io_f32 = io_dtype == HIPRWKV_F32; A.st_f32 = state_dtype == HIPRWKV_F32;
   A.flags = flags;
+  A.status = status_word();
   const bool chunked = io_dtype == HIPRWKV_BF16 && !(flags & HIPRWKV_FORCE_SEQ);
   const bool small_t = T <= HIPRWKV_SMALL_T && !(flags & HIPRWKV_NO_SMALL_T);
   hipStream_t st = static_cast<hipStream_t>(stream);
@@ -169,6 +207,7 @@ int hiprwkv_wkv6_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64
   A.length = length; A.ns = new_starts;
   A.io_f32 = io_dtype == HIPRWKV_F32; A.st_f32 = state_dtype == HIPRWKV_F32;
   A.flags = flags;
+  A.status = status_word();
   A.gy = gy; A.gs_out = gs_out;
   A.gr = gr; A.gk = gk; A.gv = gv; A.gw = gw; A.gu = gu; A.gs = gs;
   char* ws = static_cast<char*>(workspace);
@@ -197,8 +236,10 @@ int hiprwkv_wkv4_fwd(hiprwkv_stream stream, int io_dtype, int64_t B, int64_t T, 
   // the forward kernel addresses a block of 32 tokens with 32-bit byte offsets from the block's first token
   if (C > (1LL << 23)) return fail(HIPRWKV_EINVAL, "wkv4_fwd: C exceeds 2^23 channels");
   const void* req[] = {w, u, k, v, s, new_s, out};
-  for (const void* p : req)
+  for (const void* p : req) {
     if (p == nullptr) return fail(HIPRWKV_EINVAL, "wkv4_fwd: null tensor pointer");
+    if (!aligned16(p)) return fail(HIPRWKV_EINVAL, "wkv4_fwd: tensor pointers must be 16-byte aligned");
+  }
   Wkv4Args A;
   memset(&A, 0, sizeof(A));
   A.B = B; A.T = T; A.C = C;
@@ -225,8 +266,11 @@ int hiprwkv_wkv4_bwd(hiprwkv_stream stream, int io_dtype, int64_t B, int64_t T, 
   if (B * ((C + 63) / 64) > 0x7fffffffLL) return fail(HIPRWKV_EINVAL, "wkv4_bwd: B*C exceeds the grid limit");
   if (C > (1LL << 23)) return fail(HIPRWKV_EINVAL, "wkv4_bwd: C exceeds 2^23 channels");
   const void* req[] = {w, u, k, v, gy, s, gw, gu, gk, gv, gs, workspace};
-  for (const void* p : req)
+  for (const void* p : req) {
     if (p == nullptr) return fail(HIPRWKV_EINVAL, "wkv4_bwd: null tensor pointer");
+    if (!aligned16(p)) return fail(HIPRWKV_EINVAL, "wkv4_bwd: tensor pointers must be 16-byte aligned");
+  }
+  if (gs_new && !aligned16(gs_new)) return fail(HIPRWKV_EINVAL, "wkv4_bwd: tensor pointers must be 16-byte aligned");
   const size_t need = hiprwkv_wkv4_bwd_workspace_bytes(B, T, C);
   if (workspace_bytes < need)
     return fail(HIPRWKV_ENOSPACE, "wkv4_bwd: workspace has %zu bytes, %zu needed", workspace_bytes, need);
@@ -251,8 +295,10 @@ int hiprwkv_rwkv7_premix(hiprwkv_stream stream, int io_dtype, int64_t rows, int6
   if (N != 64) return fail(HIPRWKV_EINVAL, "rwkv7_premix: head size N=%lld not supported (64 only)", (long long)N);
   if (rows <= 0 || H <= 0 || (rows * H + 3) / 4 > 0x7fffffffLL) return fail(HIPRWKV_EINVAL, "rwkv7_premix: bad rows/H");
   const void* req[] = {k, a, k_k, k_a, k_out, a_out, b_out};
-  for (const void* p : req)
+  for (const void* p : req) {
     if (p == nullptr) return fail(HIPRWKV_EINVAL, "rwkv7_premix: null tensor pointer");
+    if (!aligned16(p)) return fail(HIPRWKV_EINVAL, "rwkv7_premix: tensor pointers must be 16-byte aligned");
+  }
   hipError_t e = launch_rwkv7_premix(io_dtype == HIPRWKV_F32, rows, H, k, a, k_k, k_a, k_out, a_out, b_out,
                                      static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "rwkv7_premix: %s", hipGetErrorString(e));
@@ -266,8 +312,10 @@ int hiprwkv_rwkv7_postmix(hiprwkv_stream stream, int io_dtype, int64_t rows, int
   if (N != 64) return fail(HIPRWKV_EINVAL, "rwkv7_postmix: head size N=%lld not supported (64 only)", (long long)N);
   if (rows <= 0 || H <= 0 || (rows * H + 3) / 4 > 0x7fffffffLL) return fail(HIPRWKV_EINVAL, "rwkv7_postmix: bad rows/H");
   const void* req[] = {y, r, k, v, g, ln_w, ln_b, r_k, out};
-  for (const void* p : req)
+  for (const void* p : req) {
     if (p == nullptr) return fail(HIPRWKV_EINVAL, "rwkv7_postmix: null tensor pointer");
+    if (!aligned16(p)) return fail(HIPRWKV_EINVAL, "rwkv7_postmix: tensor pointers must be 16-byte aligned");
+  }
   hipError_t e = launch_rwkv7_postmix(io_dtype == HIPRWKV_F32, rows, H, y, r, k, v, g, ln_w, ln_b, r_k, eps, out,
                                       static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "rwkv7_postmix: %s", hipGetErrorString(e));

@@ -21,26 +21,66 @@ constexpr float MIN_STEP_L2 = -1.0e4f;          // keeps the running sum finite
 constexpr float MIN_CUM_L2 = -80.0f * LOG2E;    // floor of a chunk's total log2 decay: 2^MIN_CUM_L2 = e^-80
 
 // Hand-shake words.  ready[s] = c + 1 once chunk c is complete in slot s; consumed[q][s] = c + 1 once consumer
-// q no longer reads chunk c in slot s.  Waiting is a bounded poll, so that a broken hand-shake ends the kernel
-// (with wrong results) instead of hanging the GPU.
+// q no longer reads chunk c in slot s.  Waiting is a bounded poll, so that a broken hand-shake cannot hang the GPU:
+// a waiter that gives up sets `broken` and returns false, its wave leaves its chunk loop, and after the
+// workgroup's final barrier every output of that (sequence, head) is overwritten with NaN and the library's
+// failure counter is incremented (finish_head below), so no launch returns stale data unnoticed.
 struct __attribute__((aligned(16))) Sync {
   int ready[8];
   int consumed[NCONS][8];
+  int broken;
+  int pad[3];
 };
 
-__device__ __forceinline__ void wait_ready(const Sync* sy, int slot, int want) {
+__device__ __forceinline__ bool wait_ready(Sync* sy, int slot, int want) {
   for (int spin = 0; spin < SPIN_LIMIT; ++spin) {
-    if (__hip_atomic_load(&sy->ready[slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) == want) return;
+    if (__hip_atomic_load(&sy->ready[slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) == want) return true;
     __builtin_amdgcn_s_sleep(1);
   }
+  __hip_atomic_store(&sy->broken, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  return false;
 }
-__device__ __forceinline__ void wait_consumed(const Sync* sy, int slot, int want, int lane) {
+__device__ __forceinline__ bool wait_consumed(Sync* sy, int slot, int want, int lane) {
   for (int spin = 0; spin < SPIN_LIMIT; ++spin) {
     int seen = want;
     if (lane < NCONS) seen = __hip_atomic_load(&sy->consumed[lane][slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
-    if (__ballot(seen < want) == 0ull) return;
+    if (__ballot(seen < want) == 0ull) return true;
     __builtin_amdgcn_s_sleep(1);
   }
+  __hip_atomic_store(&sy->broken, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  return false;
+}
+
+// Test hook (HIPRWKV_DEBUG_DROP_PUBLISH): the producer of the last step does not publish it, so that the consumers'
+// bounded wait runs out while every wave still ends normally.
+constexpr unsigned FLAG_DROP_PUBLISH = 0x100u;
+
+// NaN into this head's rows of a (B,T,H,64) tensor; elem = bytes per element (2: bf16, 4: fp32)
+__device__ __forceinline__ void poison_token_rows(void* base, int elem, int64_t b, int64_t h, int64_t T, int64_t H) {
+  if (base == nullptr) return;
+  const int pieces = 64 * elem / 16;
+  const uint32_t nan = elem == 2 ? 0x7fc07fc0u : 0x7fc00000u;
+  for (int64_t i = threadIdx.x; i < T * pieces; i += blockDim.x) {
+    const int64_t t = i / pieces;
+    const int pc = (int)(i % pieces);
+    char* p = static_cast<char*>(base) + ((((size_t)b * T + t) * H + h) * 64) * elem + 16 * pc;
+    *reinterpret_cast<uint4*>(p) = make_uint4(nan, nan, nan, nan);
+  }
+}
+// NaN into this head's 64x64 block of a (B,H,64,64) state tensor
+__device__ __forceinline__ void poison_state(void* base, int f32, int64_t b, int64_t h, int64_t H) {
+  if (base == nullptr) return;
+  const int elem = f32 ? 4 : 2;
+  const uint32_t nan = f32 ? 0x7fc00000u : 0x7fc07fc0u;
+  char* p = static_cast<char*>(base) + (((size_t)b * H + h) * 4096) * elem;
+  for (int i = threadIdx.x; i < 4096 * elem / 16; i += blockDim.x)
+    reinterpret_cast<uint4*>(p)[i] = make_uint4(nan, nan, nan, nan);
+}
+// After the workgroup's final barrier: did any waiter of this workgroup give up?
+__device__ __forceinline__ bool head_broken(const Sync* sy, unsigned* status) {
+  const bool broken = __hip_atomic_load(&sy->broken, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != 0;
+  if (broken && threadIdx.x == 0 && status != nullptr) atomicAdd(status, 1u);
+  return broken;
 }
 
 __device__ __forceinline__ f32x4_t mfma(const u32x4_t a, const u32x4_t b, f32x4_t c) {
@@ -144,17 +184,14 @@ struct ChunkFlags {
 // number of resets at or before in-chunk token t: the index of its segment
 __device__ __forceinline__ int seg_of(uint32_t ns, int t) { return __builtin_popcount(ns & ((2u << t) - 1u)); }
 
-// Lanes 0..16 fetch one flag each.  The load has no predicate (lanes beyond the chunk or the sequence re-read the
-// last flag they may, and without flags every lane reads a byte of `dummy`) and its result stays in a register
-// untested, so that a caller can request it a chunk ahead; chunk_flags_of drops what does not belong to the chunk
-// and makes the 17-bit mask uniform with a ballot.
-__device__ __forceinline__ uint32_t chunk_flag_fetch(const uint8_t* ns, const void* dummy, int64_t T, int64_t b,
-                                                     int64_t c0, int lane) {
+// Lanes 0..16 fetch one flag each (lanes beyond the chunk or the sequence re-read the last flag they may); the
+// ballot in chunk_flags_of drops what does not belong to the chunk and makes the 17-bit mask uniform.  Only called
+// with a non-null `ns`.
+__device__ __forceinline__ uint32_t chunk_flag_fetch(const uint8_t* ns, int64_t T, int64_t b, int64_t c0, int lane) {
   const int64_t room = T - 1 - c0 < CK ? T - 1 - c0 : CK;          // c0 <= T - 1
-  const void* base = ns != nullptr ? static_cast<const void*>(ns + (size_t)b * T + c0) : dummy;
-  const int off = ns != nullptr ? (lane < (int)room ? lane : (int)room) : 0;
+  const int off = lane < (int)room ? lane : (int)room;
   return __builtin_amdgcn_raw_buffer_load_b8(
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7fffffff, 0x00020000), off, 0, 0);
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t*>(ns + (size_t)b * T + c0), 0, 0x7fffffff, 0x00020000), off, 0, 0);
 }
 __device__ __forceinline__ ChunkFlags chunk_flags_of(const uint8_t* ns, uint32_t mine, unsigned flags, int64_t T,
                                                      int64_t c0, int64_t L) {
@@ -166,9 +203,13 @@ __device__ __forceinline__ ChunkFlags chunk_flags_of(const uint8_t* ns, uint32_t
   F.ns = ns != nullptr ? (uint32_t)(__ballot(mine != 0) & ((1ull << have) - 1ull)) : 0u;
   return F;
 }
+// Without new_starts (a null pointer is legal) nothing is loaded: the branch is uniform, the pointer is a kernel
+// argument.
 __device__ __forceinline__ ChunkFlags chunk_flags(const uint8_t* ns, unsigned flags, int64_t T, int64_t b, int64_t c0,
                                                   int64_t L, int lane) {
-  return chunk_flags_of(ns, chunk_flag_fetch(ns, ns, T, b, c0, lane), flags, T, c0, L);
+  uint32_t mine = 0u;
+  if (ns != nullptr) mine = chunk_flag_fetch(ns, T, b, c0, lane);
+  return chunk_flags_of(ns, mine, flags, T, c0, L);
 }
 
 // Selection operands that turn an MFMA into a transposer: against an A operand whose k-slot (g, jj) stands for key

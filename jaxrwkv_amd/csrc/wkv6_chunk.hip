@@ -273,7 +273,7 @@ __device__ __forceinline__ size_t state_off(const Wkv6Args& A, int64_t b, int64_
 }
 
 template <class WaitNext>
-__device__ __forceinline__ void consume(Consumer& C, Ops& o, const Slot* __restrict__ slot,
+__device__ __forceinline__ bool consume(Consumer& C, Ops& o, const Slot* __restrict__ slot,
                                         const Slot* __restrict__ next, const SnapSlot* __restrict__ snapslot,
                                         const Wkv6Args& A, int64_t b, int64_t h, int nvalid, bool is_snap, bool q2drop,
                                         OutCursor& oc, WaitNext&& next_ready) {
@@ -306,8 +306,9 @@ __device__ __forceinline__ void consume(Consumer& C, Ops& o, const Slot* __restr
   float4 gm[4];
 #pragma unroll
   for (int tile = 0; tile < 4; ++tile) gm[tile] = *reinterpret_cast<const float4*>(&slot->gamma[16 * tile + 4 * g]);
+  bool ok = true;
   if (next != nullptr) {
-    next_ready();
+    ok = next_ready();
     load_ops(o, next, C.q, lane);
   }
   // state snapshot for `length` (one chunk per sequence)
@@ -362,6 +363,7 @@ __device__ __forceinline__ void consume(Consumer& C, Ops& o, const Slot* __restr
     }
   }
   oc.y += CK * oc.tok_bytes;
+  return ok;
 }
 
 __device__ __forceinline__ void load_state(Consumer& C, const Wkv6Args& A, int64_t b, int64_t h) {
@@ -426,16 +428,17 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD), 4) void wkv6_chunk_fwd_kernel
     const int csnap = L >= 1 ? (int)((L - 1) / CK) : -1;
     const int nch = (int)nchunks;
     Ops ops;
+    bool ok = true;
     if (nch > 0) {
-      wait_ready(sy, 0, 1);
+      ok = wait_ready(sy, 0, 1);
       load_ops(ops, &slots[0], wave, lane);
     }
-    for (int c = 0; c < nch; ++c) {
+    for (int c = 0; c < nch && ok; ++c) {
       const int nvalid = (c + 1 < nch || A.T % CK == 0) ? CK : (int)(A.T % CK);
       const int si = c % RING, sn = (c + 1) % RING;
       const Slot* next = (c + 1 < nch) ? &slots[sn] : nullptr;
-      consume(C, ops, &slots[si], next, snapslot, A, b, h, nvalid, c == csnap, q2drop, oc,
-              [&]() { wait_ready(sy, sn, c + 2); });
+      ok = consume(C, ops, &slots[si], next, snapslot, A, b, h, nvalid, c == csnap, q2drop, oc,
+                   [&]() { return wait_ready(sy, sn, c + 2); });
       // every LDS read of slot si has returned: its data went into the MFMAs above
       if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], c + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
@@ -452,20 +455,26 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD), 4) void wkv6_chunk_fwd_kernel
       const ChunkFlags F = chunk_flags(A.ns, A.flags, A.T, b, c0, L, lane);
       const int si = (int)(c % RING);
       Slot* slot = &slots[si];
-      if (c >= RING) wait_consumed(sy, si, (int)(c - RING) + 1, lane);
+      if (c >= RING && !wait_consumed(sy, si, (int)(c - RING) + 1, lane)) break;
       produce(P, raw, F, slot, snapslot);
       if (c + NPROD < nchunks) load_raw(raw, A, b, h, c0 + NPROD * CK, lane);
+      if ((A.flags & FLAG_DROP_PUBLISH) && c + 1 == nchunks) break;
       // the release orders this wave's LDS writes before the sequence number
       if (lane == 0) __hip_atomic_store(&sy->ready[si], (int)c + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
+  }
+  __syncthreads();
+  if (head_broken(sy, A.status)) {
+    poison_token_rows(A.out, 2, b, h, A.T, A.H);
+    poison_state(A.new_s, A.st_f32, b, h, A.H);
   }
 }
 
 hipError_t launch_wkv6_chunk_fwd(const Wkv6Args& A, hipStream_t stream) {
   const size_t smem = RING * sizeof(Slot) + sizeof(SnapSlot) + sizeof(Sync) + 64 * sizeof(uint16_t);
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(wkv6_chunk_fwd_kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-  if (e != hipSuccess) return e;
+  static LdsAttrOnce once;
+  const hipError_t attr = allow_dynamic_lds(once, reinterpret_cast<const void*>(wkv6_chunk_fwd_kernel), smem);
+  if (attr != hipSuccess) return attr;
   hipLaunchKernelGGL(wkv6_chunk_fwd_kernel, dim3((unsigned)(A.B * A.H)), dim3(64 * (NCONS + NPROD)), smem, stream, A);
   return hipGetLastError();
 }

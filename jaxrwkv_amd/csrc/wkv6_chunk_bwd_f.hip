@@ -400,7 +400,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv6_chunk_bwd_f_kernel(
     for (int c = 0; c < nch; ++c) {
       const int nvalid = (c + 1 < nch || A.T % CK == 0) ? CK : (int)(A.T % CK);
       const int si = c % RING;
-      wait_ready(sy, si, c + 1);
+      if (!wait_ready(sy, si, c + 1)) break;
       consume(C, &slots[si], snapslot, A, b, h, nvalid, c == csnap, oc);
       if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], c + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
@@ -424,9 +424,10 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv6_chunk_bwd_f_kernel(
       if (!inject) F.snap = -1;
       const int si = c % RING;
       Slot* slot = &slots[si];
-      if (c >= RING) wait_consumed(sy, si, c - RING + 1, lane);
+      if (c >= RING && !wait_consumed(sy, si, c - RING + 1, lane)) break;
       produce(P, raw, F, slot, snapslot);
       if (c + NPROD < nch) load_raw(raw, A, b, h, c0 + NPROD * CK, lane);
+      if ((A.flags & FLAG_DROP_PUBLISH) && c + 1 == nch) break;
       if (lane == 0) __hip_atomic_store(&sy->ready[si], c + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
     // du of this producer's tokens: sum over the 16 token lanes of a row, one writer per key
@@ -443,13 +444,18 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv6_chunk_bwd_f_kernel(
     for (int p = 0; p < NPROD; ++p) s += tail->du[p][threadIdx.x];
     A.gu[((size_t)b * A.H + h) * 64 + threadIdx.x] = s;
   }
+  if (head_broken(sy, A.status)) {
+    poison_token_rows(A.gr, 2, b, h, A.T, A.H);
+    poison_token_rows(A.er, 4, b, h, A.T, A.H);
+    if (threadIdx.x < 64) A.gu[((size_t)b * A.H + h) * 64 + threadIdx.x] = __uint_as_float(0x7fc00000u);
+  }
 }
 
 hipError_t launch_wkv6_chunk_bwd_f(const Wkv6Args& A, hipStream_t stream) {
   const size_t smem = RING * sizeof(Slot) + sizeof(SnapSlot) + sizeof(Tail) + sizeof(Sync);
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(wkv6_chunk_bwd_f_kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-  if (e != hipSuccess) return e;
+  static LdsAttrOnce once;
+  const hipError_t attr = allow_dynamic_lds(once, reinterpret_cast<const void*>(wkv6_chunk_bwd_f_kernel), smem);
+  if (attr != hipSuccess) return attr;
   hipLaunchKernelGGL(wkv6_chunk_bwd_f_kernel, dim3((unsigned)(A.B * A.H)), dim3(64 * (NCONS + NPROD)), smem, stream, A);
   return hipGetLastError();
 }

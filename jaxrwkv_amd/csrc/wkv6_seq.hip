@@ -264,13 +264,10 @@ __global__ __launch_bounds__(SEQ_THREADS) void wkv6_seq_bwd_r_kernel(Wkv6Args A)
 }
 
 // ------------------------------------------------------------------ host launchers
-static hipError_t set_smem6(const void* fn, size_t bytes) {
-  return hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-}
-
 hipError_t launch_wkv6_seq_fwd(const Wkv6Args& A, hipStream_t stream) {
   constexpr size_t smem = seq_smem_bytes<4, 1, F6_CH>();
-  hipError_t e = set_smem6(reinterpret_cast<const void*>(wkv6_seq_fwd_kernel), smem);
+  static LdsAttrOnce once;
+  hipError_t e = allow_dynamic_lds(once, reinterpret_cast<const void*>(wkv6_seq_fwd_kernel), smem);
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(wkv6_seq_fwd_kernel, dim3((unsigned)(A.B * A.H)), dim3(SEQ_THREADS), smem, stream, A);
   return hipGetLastError();
@@ -279,9 +276,10 @@ hipError_t launch_wkv6_seq_fwd(const Wkv6Args& A, hipStream_t stream) {
 hipError_t launch_wkv6_seq_bwd(const Wkv6Args& A, hipStream_t stream) {
   constexpr size_t sf = seq_smem_bytes<5, 2, BF6_CH>();
   constexpr size_t sr = seq_smem_bytes<6, 3, BR6_CH>();
+  static LdsAttrOnce once_f, once_r;
   hipError_t e;
-  if ((e = set_smem6(reinterpret_cast<const void*>(wkv6_seq_bwd_f_kernel), sf)) != hipSuccess) return e;
-  if ((e = set_smem6(reinterpret_cast<const void*>(wkv6_seq_bwd_r_kernel), sr)) != hipSuccess) return e;
+  if ((e = allow_dynamic_lds(once_f, reinterpret_cast<const void*>(wkv6_seq_bwd_f_kernel), sf)) != hipSuccess) return e;
+  if ((e = allow_dynamic_lds(once_r, reinterpret_cast<const void*>(wkv6_seq_bwd_r_kernel), sr)) != hipSuccess) return e;
   const dim3 grid((unsigned)(A.B * A.H)), block(SEQ_THREADS);
   hipLaunchKernelGGL(wkv6_seq_bwd_f_kernel, grid, block, sf, stream, A);
   if ((e = hipGetLastError()) != hipSuccess) return e;

@@ -458,7 +458,7 @@ __device__ __forceinline__ void store_state_tile(void* p, int f32, size_t off, c
 // The state-dependent part of one chunk.  `next` is the slot of the chunk handled after this one (null after the
 // last one); `next_ready` waits until its producer has published it.
 template <bool REV, class WaitNext>
-__device__ __forceinline__ void consume(Consumer& C, Ops& o, const Slot* __restrict__ slot,
+__device__ __forceinline__ bool consume(Consumer& C, Ops& o, const Slot* __restrict__ slot,
                                         const Slot* __restrict__ next, const SnapSlotT<REV>* __restrict__ snapslot,
                                         const Wkv7Args& A, int64_t b, int64_t h, int nvalid, bool is_snap, bool q2drop,
                                         OutCursor& oc, WaitNext&& next_ready) {
@@ -536,8 +536,9 @@ __device__ __forceinline__ void consume(Consumer& C, Ops& o, const Slot* __restr
     }
   }
   // At, Qt, Mka, Mkr, v^T are dead now: fetch the next chunk's into the same registers
+  bool ok = true;
   if (next != nullptr) {
-    next_ready();
+    ok = next_ready();
     load_aq(o, next, C.q, lane);
   }
   uint32_t h0, l0, h1, l1;
@@ -625,6 +626,7 @@ __device__ __forceinline__ void consume(Consumer& C, Ops& o, const Slot* __restr
     oc.y -= CK * oc.tok_bytes;
     oc.sa -= 2 * CK * oc.tok_bytes;
   }
+  return ok;
 }
 
 }  // namespace
@@ -687,17 +689,18 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_kernel(Wkv7Ar
     oc.voff = (uint32_t)((4 * (lane >> 4)) * (int)A.H * 64 + 16 * wave + (lane & 15));
     const int csnap = (L >= 1 && (!REV || inject)) ? (int)((L - 1) / CK) : -1;
     Ops ops;
+    bool ok = true;
     if (nch > 0) {
-      wait_ready(sy, 0, 1);
+      ok = wait_ready(sy, 0, 1);
       load_ops(ops, &slots[0], wave, lane);
     }
-    for (int j = 0; j < nch; ++j) {
+    for (int j = 0; j < nch && ok; ++j) {
       const int c = REV ? nch - 1 - j : j;
       const int nvalid = (c + 1 < nch || A.T % CK == 0) ? CK : (int)(A.T % CK);
       const int si = j % RING, sn = (j + 1) % RING;
       const Slot* next = (j + 1 < nch) ? &slots[sn] : nullptr;
-      consume<REV>(C, ops, &slots[si], next, snapslot, A, b, h, nvalid, c == csnap, q2drop, oc,
-                   [&]() { wait_ready(sy, sn, j + 2); });
+      ok = consume<REV>(C, ops, &slots[si], next, snapslot, A, b, h, nvalid, c == csnap, q2drop, oc,
+                        [&]() { return wait_ready(sy, sn, j + 2); });
       // every LDS read of slot si has returned: its data went into the MFMAs above
       if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
@@ -726,12 +729,25 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_kernel(Wkv7Ar
       if (REV && !inject) F.snap = -1;
       const int si = j % RING;
       Slot* slot = &slots[si];
-      if (j >= RING) wait_consumed(sy, si, j - RING + 1, lane);
+      if (j >= RING && !wait_consumed(sy, si, j - RING + 1, lane)) break;
       mask_raw(raw, F.nvalid, lane);
       produce<REV>(P, raw, F, slot, snapslot);
       if (j + NPROD < nch) load_raw<REV>(raw, A, b, h, (int64_t)(REV ? c - NPROD : c + NPROD) * CK, lane);
+      if ((A.flags & FLAG_DROP_PUBLISH) && j + 1 == nch) break;
       // the release orders this wave's LDS writes before the sequence number
       if (lane == 0) __hip_atomic_store(&sy->ready[si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+  }
+  __syncthreads();
+  if (head_broken(sy, A.status)) {
+    if constexpr (!REV) {
+      poison_token_rows(A.out, 2, b, h, A.T, A.H);
+      poison_token_rows(A.sa, 4, b, h, A.T, A.H);
+      poison_state(A.new_s, A.st_f32, b, h, A.H);
+    } else {
+      poison_token_rows(A.gv, 2, b, h, A.T, A.H);
+      poison_token_rows(A.dsa, 4, b, h, A.T, A.H);
+      poison_state(A.gs, A.st_f32, b, h, A.H);
     }
   }
 }
@@ -739,9 +755,9 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_kernel(Wkv7Ar
 template <bool REV>
 static hipError_t launch_chunk(const Wkv7Args& A, hipStream_t stream) {
   const size_t smem = RING * sizeof(Slot) + sizeof(SnapSlotT<REV>) + sizeof(Sync);
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(wkv7_chunk_kernel<REV>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-  if (e != hipSuccess) return e;
+  static LdsAttrOnce once;
+  const hipError_t attr = allow_dynamic_lds(once, reinterpret_cast<const void*>(wkv7_chunk_kernel<REV>), smem);
+  if (attr != hipSuccess) return attr;
   hipLaunchKernelGGL(wkv7_chunk_kernel<REV>, dim3((unsigned)(A.B * A.H)), dim3(64 * (NCONS + NPROD)), smem, stream, A);
   return hipGetLastError();
 }

@@ -498,7 +498,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_bwd_b_kernel(
     for (int c = 0; c < nch; ++c) {
       const int nvalid = (c + 1 < nch || A.T % CK == 0) ? CK : (int)(A.T % CK);
       const int si = c % RING;
-      wait_ready(sy, si, c + 1);
+      if (!wait_ready(sy, si, c + 1)) break;
       consume(C, &slots[si], snapslot, A, b, h, nvalid, c == csnap, c == 0, c + 1 == nch, oc);
       // every LDS read of slot si has returned: its data went into the MFMAs and stores above
       if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], c + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -516,20 +516,27 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_bwd_b_kernel(
       if (!inject) F.snap = -1;
       const int si = c % RING;
       Slot* slot = &slots[si];
-      if (c >= RING) wait_consumed(sy, si, c - RING + 1, lane);
+      if (c >= RING && !wait_consumed(sy, si, c - RING + 1, lane)) break;
       produce(P, raw, F, slot, snapslot);
       if (c + NPROD < nch) load_raw(raw, A, b, h, c0 + NPROD * CK, lane);
+      if ((A.flags & FLAG_DROP_PUBLISH) && c + 1 == nch) break;
       // the release orders this wave's LDS writes before the sequence number
       if (lane == 0) __hip_atomic_store(&sy->ready[si], c + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
+  }
+  __syncthreads();
+  if (head_broken(sy, A.status)) {
+    poison_token_rows(A.gr, 2, b, h, A.T, A.H);
+    poison_token_rows(A.ga, 2, b, h, A.T, A.H);
+    poison_token_rows(A.e2, 4, b, h, A.T, A.H);
   }
 }
 
 hipError_t launch_wkv7_chunk_bwd_b(const Wkv7Args& A, hipStream_t stream) {
   const size_t smem = RING * sizeof(Slot) + sizeof(SnapSlot) + sizeof(Sync);
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(wkv7_chunk_bwd_b_kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-  if (e != hipSuccess) return e;
+  static LdsAttrOnce once;
+  const hipError_t attr = allow_dynamic_lds(once, reinterpret_cast<const void*>(wkv7_chunk_bwd_b_kernel), smem);
+  if (attr != hipSuccess) return attr;
   hipLaunchKernelGGL(wkv7_chunk_bwd_b_kernel, dim3((unsigned)(A.B * A.H)), dim3(64 * (NCONS + NPROD)), smem, stream, A);
   return hipGetLastError();
 }

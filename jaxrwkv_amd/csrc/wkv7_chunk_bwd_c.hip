@@ -539,21 +539,22 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_bwd_c_kernel(
     const int tail = (A.T % CK == 0) ? CK : (int)(A.T % CK);
     Pre pre_a, pre_b;
     if (nch > 0) prefetch(pre_a, cu, tail, g);
-    auto step = [&](int j, const Pre& pre, Pre& pre_next) {
+    auto step = [&](int j, const Pre& pre, Pre& pre_next) -> bool {
       const int c = nch - 1 - j;
       const int nvalid = (j == 0) ? tail : CK;
       const int si = j % RING;
       Cursor nxt = cu;
       step_back(nxt);
-      wait_ready(sy, si, j + 1);
+      if (!wait_ready(sy, si, j + 1)) return false;
       consume(C, &slots[si], snapslot, A, b, h, nvalid, c == csnap, pre, pre_next, cu, nxt, j + 1 < nch);
       cu = nxt;
       // every LDS read of slot si has returned: its data went into the MFMAs and stores above
       if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+      return true;
     };
     for (int j = 0; j < nch; j += 2) {      // two steps per turn: the prefetch registers alternate
-      step(j, pre_a, pre_b);
-      if (j + 1 < nch) step(j + 1, pre_b, pre_a);
+      if (!step(j, pre_a, pre_b)) break;
+      if (j + 1 < nch && !step(j + 1, pre_b, pre_a)) break;
     }
   } else {
     const int p = wave - NCONS;
@@ -569,20 +570,27 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_bwd_c_kernel(
       if (!inject) F.snap = -1;
       const int si = j % RING;
       Slot* slot = &slots[si];
-      if (j >= RING) wait_consumed(sy, si, j - RING + 1, lane);
+      if (j >= RING && !wait_consumed(sy, si, j - RING + 1, lane)) break;
       produce(P, raw, F, slot, snapslot);
       if (j + NPROD < nch) load_raw(raw, A, b, h, (int64_t)(c - NPROD) * CK, lane);
+      if ((A.flags & FLAG_DROP_PUBLISH) && j + 1 == nch) break;
       // the release orders this wave's LDS writes before the sequence number
       if (lane == 0) __hip_atomic_store(&sy->ready[si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
+  }
+  __syncthreads();
+  if (head_broken(sy, A.status)) {
+    poison_token_rows(A.gk, 2, b, h, A.T, A.H);
+    poison_token_rows(A.gb, 2, b, h, A.T, A.H);
+    poison_token_rows(A.gw, 2, b, h, A.T, A.H);
   }
 }
 
 hipError_t launch_wkv7_chunk_bwd_c(const Wkv7Args& A, hipStream_t stream) {
   const size_t smem = RING * sizeof(Slot) + sizeof(SnapSlot) + sizeof(Sync);
-  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(wkv7_chunk_bwd_c_kernel),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-  if (e != hipSuccess) return e;
+  static LdsAttrOnce once;
+  const hipError_t attr = allow_dynamic_lds(once, reinterpret_cast<const void*>(wkv7_chunk_bwd_c_kernel), smem);
+  if (attr != hipSuccess) return attr;
   hipLaunchKernelGGL(wkv7_chunk_bwd_c_kernel, dim3((unsigned)(A.B * A.H)), dim3(64 * (NCONS + NPROD)), smem, stream, A);
   return hipGetLastError();
 }

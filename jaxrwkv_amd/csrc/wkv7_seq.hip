@@ -321,13 +321,10 @@ __global__ __launch_bounds__(SEQ_THREADS) void wkv7_seq_bwd_c_kernel(Wkv7Args A)
 }
 
 // ------------------------------------------------------------------ host launchers
-static hipError_t set_smem(const void* fn, size_t bytes) {
-  return hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-}
-
 hipError_t launch_wkv7_seq_fwd(const Wkv7Args& A, hipStream_t stream) {
   constexpr size_t smem = seq_smem_bytes<6, 2, FWD_CH>();
-  hipError_t e = set_smem(reinterpret_cast<const void*>(wkv7_seq_fwd_kernel), smem);
+  static LdsAttrOnce once;
+  hipError_t e = allow_dynamic_lds(once, reinterpret_cast<const void*>(wkv7_seq_fwd_kernel), smem);
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(wkv7_seq_fwd_kernel, dim3((unsigned)(A.B * A.H)), dim3(SEQ_THREADS), smem, stream, A);
   return hipGetLastError();
@@ -336,7 +333,8 @@ hipError_t launch_wkv7_seq_fwd(const Wkv7Args& A, hipStream_t stream) {
 // The three backward sweeps, in the order they must run (A, B, C).
 hipError_t launch_wkv7_seq_bwd_a(const Wkv7Args& A, hipStream_t stream) {
   constexpr size_t smem = seq_smem_bytes<6, 2, BWA_CH>();
-  hipError_t e = set_smem(reinterpret_cast<const void*>(wkv7_seq_bwd_a_kernel), smem);
+  static LdsAttrOnce once;
+  hipError_t e = allow_dynamic_lds(once, reinterpret_cast<const void*>(wkv7_seq_bwd_a_kernel), smem);
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(wkv7_seq_bwd_a_kernel, dim3((unsigned)(A.B * A.H)), dim3(SEQ_THREADS), smem, stream, A);
   return hipGetLastError();
@@ -344,7 +342,8 @@ hipError_t launch_wkv7_seq_bwd_a(const Wkv7Args& A, hipStream_t stream) {
 
 hipError_t launch_wkv7_seq_bwd_b(const Wkv7Args& A, hipStream_t stream) {
   constexpr size_t smem = seq_smem_bytes<9, 4, BWB_CH>();
-  hipError_t e = set_smem(reinterpret_cast<const void*>(wkv7_seq_bwd_b_kernel), smem);
+  static LdsAttrOnce once;
+  hipError_t e = allow_dynamic_lds(once, reinterpret_cast<const void*>(wkv7_seq_bwd_b_kernel), smem);
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(wkv7_seq_bwd_b_kernel, dim3((unsigned)(A.B * A.H)), dim3(SEQ_THREADS), smem, stream, A);
   return hipGetLastError();
@@ -352,7 +351,8 @@ hipError_t launch_wkv7_seq_bwd_b(const Wkv7Args& A, hipStream_t stream) {
 
 hipError_t launch_wkv7_seq_bwd_c(const Wkv7Args& A, hipStream_t stream) {
   constexpr size_t smem = seq_smem_bytes<12, 3, BWC_CH>();
-  hipError_t e = set_smem(reinterpret_cast<const void*>(wkv7_seq_bwd_c_kernel), smem);
+  static LdsAttrOnce once;
+  hipError_t e = allow_dynamic_lds(once, reinterpret_cast<const void*>(wkv7_seq_bwd_c_kernel), smem);
   if (e != hipSuccess) return e;
   hipLaunchKernelGGL(wkv7_seq_bwd_c_kernel, dim3((unsigned)(A.B * A.H)), dim3(SEQ_THREADS), smem, stream, A);
   return hipGetLastError();

@@ -3,6 +3,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace hiprwkv {
 
 struct Wkv7Args {
@@ -21,6 +23,7 @@ struct Wkv7Args {
   const void* gs_out;
   void *gw, *gr, *gk, *gv, *ga, *gb, *gs;
   float *dsa, *e2, *e3;  // workspace, (B,T,H,64) fp32 each (the chunked sweeps keep e3_t + e2_{t+1} in e2, e3 unused)
+  unsigned* status;      // device word counting workgroups whose hand-shake gave up (may be null)
 };
 
 struct Wkv6Args {
@@ -39,6 +42,7 @@ struct Wkv6Args {
   float* gu;   // (B,H,64)
   float* er;   // workspace (B,T,H,64): r . (S' dy)
   float* eI;   // workspace (B,H,64): rowsum(dS_out * S_{length-1})
+  unsigned* status;   // device word counting workgroups whose hand-shake gave up (may be null)
 };
 
 struct Wkv4Args {
@@ -57,6 +61,22 @@ struct Wkv4Args {
   float *gw, *gu;   // (B,C) each
   float* ckpt;      // workspace: (B, ceil(T/16), 3, C) states entering every 16th step
 };
+
+// Raises a kernel's dynamic-LDS limit once per kernel and device instead of at every enqueue (the attribute call
+// goes to the driver; hipGetDevice does not).
+struct LdsAttrOnce {
+  std::atomic<uint64_t> done{0};   // bit d: set on device d
+};
+inline hipError_t allow_dynamic_lds(LdsAttrOnce& once, const void* kernel, size_t bytes) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return e;
+  const uint64_t bit = 1ull << (dev & 63);
+  if (once.done.load(std::memory_order_acquire) & bit) return hipSuccess;
+  e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (e == hipSuccess) once.done.fetch_or(bit, std::memory_order_release);
+  return e;
+}
 
 hipError_t launch_wkv7_seq_fwd(const Wkv7Args& A, hipStream_t stream);
 hipError_t launch_wkv7_chunk_fwd(const Wkv7Args& A, hipStream_t stream);

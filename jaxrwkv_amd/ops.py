@@ -45,14 +45,24 @@ def _length_ns(length, new_starts, B, T, device):
     return length, new_starts
 
 
-def _flags(compat, force_seq=False, small_t=True):
+def _flags(compat, force_seq=False, small_t=True, debug=0):
     return ((_lib.COMPAT_ASSOC if compat else 0) | (_lib.FORCE_SEQ if force_seq else 0)
-            | (0 if small_t else _lib.NO_SMALL_T))
+            | (0 if small_t else _lib.NO_SMALL_T) | int(debug))
+
+
+def handshake_failures():
+    """Workgroups of the chunked kernels whose bounded hand-shake wait ran out since the library was loaded (their
+    outputs are NaN).  Synchronises the current stream."""
+    import ctypes
+    lib = _lib.load()
+    n = ctypes.c_uint(0)
+    _lib.check(lib.hiprwkv_handshake_failures(_stream(), ctypes.byref(n)), "hiprwkv_handshake_failures")
+    return int(n.value)
 
 
 # ----------------------------------------------------------------------------- WKV7
 def wkv7_fwd(r, w, k, v, a, b, s, length=None, new_starts=None, compat=True, want_sa=False, force_seq=False,
-             small_t=True):
+             small_t=True, debug_flags=0):
     """r,w,k,v,a,b (B,T,H,N) fp32|bf16; s (B,H,N,N) fp32|bf16.  Returns (new_s, y, sa|None).
 
     T <= 8 runs on the small-T (decode) kernel unless ``small_t=False``; otherwise bf16 I/O runs on the chunked MFMA
@@ -69,12 +79,13 @@ def wkv7_fwd(r, w, k, v, a, b, s, length=None, new_starts=None, compat=True, wan
     sa = torch.empty((B, T, H, N), dtype=torch.float32, device=r.device) if want_sa else None
     rc = lib.hiprwkv_wkv7_fwd(_stream(), _DT[io], _DT[s.dtype], B, T, H, N, _p(w), _p(r), _p(k), _p(v), _p(a), _p(b),
                               _p(s), _p(length), _p(new_starts), _p(y), _p(sa), _p(new_s),
-                              _flags(compat, force_seq, small_t))
+                              _flags(compat, force_seq, small_t, debug_flags))
     _lib.check(rc, "hiprwkv_wkv7_fwd")
     return new_s, y, sa
 
 
-def wkv7_bwd(r, w, k, v, a, b, s, length, new_starts, gy, sa, gs_out=None, compat=True, force_seq=False):
+def wkv7_bwd(r, w, k, v, a, b, s, length, new_starts, gy, sa, gs_out=None, compat=True, force_seq=False,
+             debug_flags=0):
     """Cotangents (gr, gw, gk, gv, ga, gb, gs) of ``wkv7_fwd`` for cotangents gy of y and gs_out of new_s.
 
     bf16 inputs use the chunked MFMA kernels where they exist unless ``force_seq`` asks for the sequential ones."""
@@ -93,7 +104,7 @@ def wkv7_bwd(r, w, k, v, a, b, s, length, new_starts, gy, sa, gs_out=None, compa
     rc = lib.hiprwkv_wkv7_bwd(_stream(), _DT[io], _DT[s.dtype], B, T, H, N, _p(w), _p(r), _p(k), _p(v), _p(a), _p(b),
                               _p(s), _p(length), _p(new_starts), _p(gy), _p(sa), _p(gs_out),
                               _p(gw), _p(gr), _p(gk), _p(gv), _p(ga), _p(gb), _p(gs), _p(ws), nbytes,
-                              _flags(compat, force_seq))
+                              _flags(compat, force_seq, debug=debug_flags))
     _lib.check(rc, "hiprwkv_wkv7_bwd")
     return gr, gw, gk, gv, ga, gb, gs
 
@@ -102,10 +113,11 @@ class _Wkv7(torch.autograd.Function):
     """custom VJP, the counterpart of ``wkv7_cuda`` (rwkv7.py:442-446)."""
 
     @staticmethod
-    def forward(ctx, r, w, k, v, a, b, s, length, new_starts, compat):
+    def forward(ctx, r, w, k, v, a, b, s, length, new_starts, compat, force_seq):
         need = any(x.requires_grad for x in (r, w, k, v, a, b, s))
-        new_s, y, sa = wkv7_fwd(r, w, k, v, a, b, s, length, new_starts, compat, want_sa=need)
+        new_s, y, sa = wkv7_fwd(r, w, k, v, a, b, s, length, new_starts, compat, want_sa=need, force_seq=force_seq)
         ctx.compat = compat
+        ctx.force_seq = force_seq
         ctx.save_for_backward(r, w, k, v, a, b, s, length, new_starts, sa)
         return new_s, y
 
@@ -114,19 +126,21 @@ class _Wkv7(torch.autograd.Function):
         r, w, k, v, a, b, s, length, new_starts, sa = ctx.saved_tensors
         if gy is None:
             gy = torch.zeros_like(r)
-        gr, gw, gk, gv, ga, gb, gs = wkv7_bwd(r, w, k, v, a, b, s, length, new_starts, gy, sa, gs_out, ctx.compat)
-        return gr, gw, gk, gv, ga, gb, gs, None, None, None
+        gr, gw, gk, gv, ga, gb, gs = wkv7_bwd(r, w, k, v, a, b, s, length, new_starts, gy, sa, gs_out, ctx.compat,
+                                              ctx.force_seq)
+        return gr, gw, gk, gv, ga, gb, gs, None, None, None, None
 
 
-def wkv7(r, w, k, v, a, b, s, length=None, new_starts=None, compat=True):
-    """Differentiable WKV7: returns (new_s, y)."""
+def wkv7(r, w, k, v, a, b, s, length=None, new_starts=None, compat=True, force_seq=False):
+    """Differentiable WKV7: returns (new_s, y).  ``force_seq`` runs the sequential fp32 kernels whatever the dtype."""
     B, T = r.shape[:2]
     length, new_starts = _length_ns(length, new_starts, B, T, r.device)
-    return _Wkv7.apply(r, w, k, v, a, b, s, length, new_starts, compat)
+    return _Wkv7.apply(r, w, k, v, a, b, s, length, new_starts, compat, force_seq)
 
 
 # ----------------------------------------------------------------------------- WKV6
-def wkv6_fwd(r, k, v, w, u, s, length=None, new_starts=None, compat=True, force_seq=False, small_t=True):
+def wkv6_fwd(r, k, v, w, u, s, length=None, new_starts=None, compat=True, force_seq=False, small_t=True,
+             debug_flags=0):
     """r,k,v,w (B,T,H,N); u (H,N); s (B,H,N,N) [key, value].  Returns (new_s, y).
 
     T <= 8 runs on the small-T (decode) kernel unless ``small_t=False``; otherwise bf16 inputs run on the chunked
@@ -143,12 +157,12 @@ def wkv6_fwd(r, k, v, w, u, s, length=None, new_starts=None, compat=True, force_
     new_s = torch.empty_like(s)
     rc = lib.hiprwkv_wkv6_fwd(_stream(), _DT[io], _DT[s.dtype], B, T, H, N, _p(r), _p(k), _p(v), _p(w), _p(u), _p(s),
                               _p(length), _p(new_starts), _p(y), _p(new_s),
-                              _flags(compat, force_seq, small_t))
+                              _flags(compat, force_seq, small_t, debug_flags))
     _lib.check(rc, "hiprwkv_wkv6_fwd")
     return new_s, y
 
 
-def wkv6_bwd(r, k, v, w, u, s, length, new_starts, gy, gs_out=None, compat=True, force_seq=False):
+def wkv6_bwd(r, k, v, w, u, s, length, new_starts, gy, gs_out=None, compat=True, force_seq=False, debug_flags=0):
     """Cotangents (gr, gk, gv, gw, gu, gs) of ``wkv6_fwd``; gu is summed over the batch here.
 
     bf16 inputs run on the chunked MFMA kernels unless ``force_seq`` asks for the sequential fp32 ones."""
@@ -168,7 +182,7 @@ def wkv6_bwd(r, k, v, w, u, s, length, new_starts, gy, gs_out=None, compat=True,
     ws = torch.empty(nbytes, dtype=torch.uint8, device=r.device)
     rc = lib.hiprwkv_wkv6_bwd(_stream(), _DT[io], _DT[s.dtype], B, T, H, N, _p(r), _p(k), _p(v), _p(w), _p(u), _p(s),
                               _p(length), _p(new_starts), _p(gy), _p(gs_out), _p(gr), _p(gk), _p(gv), _p(gw), _p(gu),
-                              _p(gs), _p(ws), nbytes, _flags(compat, force_seq))
+                              _p(gs), _p(ws), nbytes, _flags(compat, force_seq, debug=debug_flags))
     _lib.check(rc, "hiprwkv_wkv6_bwd")
     return gr, gk, gv, gw, gu.sum(0).to(io), gs
 

@@ -16,6 +16,8 @@ from . import ops
 class HipRWKV:
     #: True -> results equal AssociativeScanRWKV (rwkv7.py:321-346); False -> BaseRWKV/ScanRWKV (rwkv7.py:200-220)
     assoc_compat = True
+    #: True -> the sequential fp32 kernels whatever the dtype (the cross-check of the chunked MFMA kernels)
+    force_seq = False
 
     @classmethod
     def inner_loop(cls, r, w, k, v, a, b, s, length, new_starts):
@@ -27,7 +29,7 @@ class HipRWKV:
             r, w, k, v, a, b, s = (x[None] for x in (r, w, k, v, a, b, s))
             if torch.is_tensor(new_starts) and new_starts.dim() == 1:
                 new_starts = new_starts[None]
-        new_s, y = ops.wkv7(r, w, k, v, a, b, s, length, new_starts, cls.assoc_compat)
+        new_s, y = ops.wkv7(r, w, k, v, a, b, s, length, new_starts, cls.assoc_compat, cls.force_seq)
         new_s = new_s.to(r.dtype)
         if not batched:
             new_s, y = new_s[0], y[0]

@@ -54,6 +54,26 @@ def test_argument_validation_without_gpu():
     assert lib.hiprwkv_wkv6_bwd_workspace_bytes(2, 16, 2, 64) >= 2 * 16 * 2 * 64 * 4
 
 
+def test_misaligned_pointers_are_refused_by_every_entry_point():
+    """All tensor pointers must be 16-byte aligned (the kernels use 8- and 16-byte accesses); refused before a launch."""
+    from jaxrwkv_amd import _lib
+    lib = _lib.load()
+    ok, bad, null = ctypes.c_void_p(0x10000), ctypes.c_void_p(0x10008), ctypes.c_void_p(0)
+    msg = lambda: lib.hiprwkv_last_error()
+    rc = lib.hiprwkv_wkv7_fwd(null, 1, 0, 1, 32, 1, 64, ok, ok, bad, ok, ok, ok, ok, null, null, ok, null, ok, 0)
+    assert rc == -1 and b"aligned" in msg()
+    rc = lib.hiprwkv_wkv6_fwd(null, 1, 0, 1, 32, 1, 64, ok, ok, ok, bad, ok, ok, null, null, ok, ok, 0)
+    assert rc == -1 and b"aligned" in msg()
+    rc = lib.hiprwkv_wkv4_fwd(null, 0, 1, 8, 64, ok, ok, bad, ok, ok, null, null, ok, ok, 0)
+    assert rc == -1 and b"aligned" in msg()
+    rc = lib.hiprwkv_wkv4_bwd(null, 0, 1, 8, 64, ok, ok, ok, ok, ok, ok, null, null, null, ok, ok, ok, bad, ok, ok, 1 << 20, 0)
+    assert rc == -1 and b"aligned" in msg()
+    rc = lib.hiprwkv_rwkv7_premix(null, 1, 8, 1, 64, ok, ok, ok, ok, ok, bad, ok)
+    assert rc == -1 and b"aligned" in msg()
+    rc = lib.hiprwkv_rwkv7_postmix(null, 1, 8, 1, 64, ok, bad, ok, ok, ok, ok, ok, ok, 1e-5, ok)
+    assert rc == -1 and b"aligned" in msg()
+
+
 def test_cpu_tensors_are_refused_loudly():
     from jaxrwkv_amd import _lib, ops
     x = torch.zeros(1, 4, 1, 64)

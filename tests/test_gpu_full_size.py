@@ -12,7 +12,7 @@ def rel_rms(a, b):
     return float((a - b).pow(2).mean().sqrt() / b.pow(2).mean().sqrt().clamp_min(1e-30))
 
 
-def wkv7_full(B=8, T=4096, H=32, N=64, seed=0):
+def wkv7_full(B=8, T=4096, H=32, N=64, seed=0, p_reset=1.0 / 1024):
     g = torch.Generator("cuda").manual_seed(seed)
     n = lambda *s: torch.randn(s, device="cuda", generator=g)
     r, k, v, dy = (n(B, T, H, N).bfloat16() for _ in range(4))
@@ -20,7 +20,7 @@ def wkv7_full(B=8, T=4096, H=32, N=64, seed=0):
     kap = torch.nn.functional.normalize(n(B, T, H, N), dim=-1)
     a, b = (-kap).bfloat16(), (kap * torch.sigmoid(n(B, T, H, N))).bfloat16()
     s = 0.1 * n(B, H, N, N)
-    ns = torch.rand((B, T), device="cuda", generator=g) < 1.0 / 1024
+    ns = torch.rand((B, T), device="cuda", generator=g) < p_reset
     length = torch.randint(T // 2, T + 1, (B,), device="cuda", generator=g, dtype=torch.int32)
     return dict(r=r, w=w, k=k, v=v, a=a, b=b, s=s, ns=ns, length=length, dy=dy)
 
@@ -108,3 +108,54 @@ def test_wkv4_split_call_equals_single_call_at_the_benchmark_shape():
     torch.cuda.synchronize()
     assert torch.equal(torch.cat([y1, y2], 1), full_y)
     assert torch.equal(s2, full_s)
+
+
+def test_wkv7_prefill_shape_of_the_1p5b_config():
+    """BASELINE configs[4], prefill: the op at B=16, T=4096, H=32, bf16, new_starts ~ Bernoulli(1/2048).  Chunked
+    against sequential kernel, and a split call with the carried state against the single call."""
+    from jaxrwkv_amd import ops
+    x = wkv7_full(B=16, seed=5, p_reset=1.0 / 2048)
+    args = [x[n] for n in "rwkvab"]
+    new_s, y, _ = ops.wkv7_fwd(*args, x["s"], x["length"], x["ns"], compat=True)
+    seq_s, seq_y, _ = ops.wkv7_fwd(*args, x["s"], x["length"], x["ns"], compat=True, force_seq=True)
+    torch.cuda.synchronize()
+    assert torch.isfinite(y.float()).all() and torch.isfinite(new_s).all()
+    assert rel_rms(y, seq_y) < 4e-3, rel_rms(y, seq_y)
+    assert rel_rms(new_s, seq_s) < 2e-3, rel_rms(new_s, seq_s)
+    # y is exactly zero where the associative form defines it so, in both kernels
+    nxt = torch.zeros_like(x["ns"])
+    nxt[:, :-1] = x["ns"][:, 1:]
+    assert torch.count_nonzero(y[nxt]) == 0 and torch.count_nonzero(seq_y[nxt]) == 0
+    del seq_s, seq_y
+    full_s, full_y, _ = ops.wkv7_fwd(*args, x["s"], None, x["ns"], compat=False)
+    h = 2048
+    sl = lambda t, a, b: t[:, a:b].contiguous()
+    s1, y1, _ = ops.wkv7_fwd(*(sl(t, 0, h) for t in args), x["s"], None, sl(x["ns"], 0, h), compat=False)
+    s2, y2, _ = ops.wkv7_fwd(*(sl(t, h, 4096) for t in args), s1, None, sl(x["ns"], h, 4096), compat=False)
+    torch.cuda.synchronize()
+    assert torch.equal(torch.cat([y1, y2], 1), full_y)
+    assert torch.equal(s2, full_s)
+
+
+@pytest.mark.parametrize("st", [torch.float32, torch.bfloat16])
+def test_wkv7_decode_shape_of_the_1p5b_config(st):
+    """BASELINE configs[4], decode: one token for B=256 sequences x 32 heads from a carried state, against the float64
+    oracle (bf16 inputs; fp32 state to the fp32 bar, bf16 state and y within one bf16 ulp)."""
+    import numpy as np
+    from jaxrwkv_amd import ops
+    from oracle import wkv7 as o7
+    from tests.gpu_util import assert_close, dev, host
+    from tests.inputs import bf16_round, wkv7_inputs
+    x = wkv7_inputs(256, 1, 32, 64, seed=9, bf16=True, resets=False, lengths=False, s_scale=1.0)
+    x["new_starts"][::7, 0] = True                                  # some sequences start afresh at this token
+    if st == torch.bfloat16:
+        x["s"] = bf16_round(x["s"]).astype(np.float64)
+    ref_s, ref_y = o7.wkv7_base(*[x[n] for n in "rwkvab"], x["s"], x["length"], x["new_starts"], compat=True)
+    t = {n: dev(x[n], torch.bfloat16) for n in "rwkvab"}
+    new_s, y, _ = ops.wkv7_fwd(*[t[n] for n in "rwkvab"], dev(x["s"], st), dev(x["length"]), dev(x["new_starts"]), compat=True)
+    torch.cuda.synchronize()
+    assert_close("y", host(y), ref_y, rtol=2.0 ** -8, atol=1e-5)
+    if st == torch.float32:
+        assert_close("new_s", host(new_s), ref_s)
+    else:
+        assert_close("new_s", host(new_s), ref_s, rtol=2.0 ** -8, atol=1e-6)

@@ -137,3 +137,54 @@ def test_backward_length_zero_and_default_state():
         got = run_bwd(x, gy, gs, compat)
         for name, g_, rf in zip(("w", "u", "k", "v", "s"), got, (gw.sum(0), gu.sum(0), gk, gv, gsi)):
             assert_close("g" + name, g_, rf, rtol=1e-4, atol=2e-5, scale_atol=True)
+
+
+def bf16_inputs(B, T, C, seed):
+    """Inputs and state rounded to bf16, so that the float64 oracle and the kernel start from the same numbers."""
+    from tests.inputs import bf16_round
+    x = wkv4_inputs(B, T, C, seed=seed, p_reset=0.04, default_state=False, min_len=1)
+    for n in ("w", "u", "k", "v", "s"):
+        x[n] = bf16_round(x[n]).astype(np.float64)
+    if T > 4:
+        x["length"][0] = T // 2
+        x["new_starts"][0, T // 2] = True
+    return x
+
+
+@pytest.mark.parametrize("compat", [True, False])
+@pytest.mark.parametrize("B,T,C,seed", [(2, 40, 64, 41), (3, 130, 100, 42), (2, 515, 257, 43)])
+def test_bf16_forward(B, T, C, seed, compat):
+    """bf16 I/O (the reference's wkv4-fwd-bf16 target, rwkv4.py:396-397): fp32 arithmetic on bf16 inputs, outputs and
+    state rounded once: within one bf16 ulp (2^-8 relative) of the float64 oracle."""
+    x = bf16_inputs(B, T, C, seed)
+    ref_s, ref_y = o4.wkv4_ffi(x["w"], x["u"], x["k"], x["v"], x["s"], x["length"], x["new_starts"], compat=compat)
+    new_s, y = run_fwd(x, compat, torch.bfloat16)
+    assert_close("y", y, ref_y, rtol=2.0 ** -8, atol=1e-6)
+    assert_close("aa", new_s[:, 0], ref_s[:, 0], rtol=2.0 ** -8, atol=1e-6)
+    assert_close("bb", new_s[:, 1], ref_s[:, 1], rtol=2.0 ** -8, atol=1e-6)
+    big = ref_s[:, 2] < -1e29
+    assert np.array_equal(new_s[:, 2] < -1e29, big)
+    assert_close("pp", new_s[:, 2][~big], ref_s[:, 2][~big], rtol=2.0 ** -8, atol=1e-6)
+
+
+@pytest.mark.parametrize("compat", [True, False])
+@pytest.mark.parametrize("B,T,C,seed", [(2, 40, 64, 51), (3, 130, 100, 52)])
+def test_bf16_backward(B, T, C, seed, compat):
+    """bf16 I/O backward (wkv4-bwd-bf16, rwkv4.py:398-399): cotangents of k, v, s within a bf16 ulp plus 1e-3 of their
+    rms; gw, gu (fp32 per sequence, summed over B on the host, then rounded to bf16) likewise."""
+    from jaxrwkv_amd import ops
+    from tests.inputs import bf16_round
+    x = bf16_inputs(B, T, C, seed)
+    g = np.random.default_rng(seed)
+    gy = bf16_round(g.standard_normal(x["k"].shape)).astype(np.float64)
+    gs = bf16_round(g.standard_normal(x["s"].shape)).astype(np.float64)
+    ref_s, _ = o4.wkv4_ffi(x["w"], x["u"], x["k"], x["v"], x["s"], x["length"], x["new_starts"], compat=compat)
+    gs_eff = np.where(ref_s > -1e29, gs, 0.0)
+    ref = o4.wkv4_ffi_bwd(x["w"], x["u"], x["k"], x["v"], x["s"], x["length"], x["new_starts"], gy, gs_eff, compat=compat)
+    bf = torch.bfloat16
+    got = ops.wkv4_bwd(dev(x["w"], bf), dev(x["u"], bf), dev(x["k"], bf), dev(x["v"], bf), dev(x["s"], bf),
+                       dev(x["length"]), dev(x["new_starts"]), dev(gy, bf), dev(gs_eff, bf), compat=compat)
+    torch.cuda.synchronize()
+    gw, gu, gk, gv, gsi = ref
+    for name, g_, rf in zip(("w", "u", "k", "v", "s"), got, (gw.sum(0), gu.sum(0), gk, gv, gsi)):
+        assert_close("g" + name, host(g_), rf, rtol=2.0 ** -7, atol=1e-3, scale_atol=True)

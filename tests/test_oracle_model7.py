@@ -70,3 +70,153 @@ def test_reference_initialisation_makes_blocks_vanish():
     x = om.layer_norm(m["emb"]["weight"][t], m["ln0"])
     np.testing.assert_allclose(logits, om.layer_norm(x, m["ln_out"]) @ m["head"]["weight"].T, rtol=1e-12, atol=1e-12)
     assert np.abs(state[:, 2:]).max() > 0          # the recurrence still ran
+
+
+# ---- special cases that pin the formulas of time_mixing_seq / channel_mixing_seq (rwkv7.py:190-198, 223-267): a
+#      wrong sign in the decay, exchanged k_k / k_a, a wrong v_first mix or bonus term fails one of them.  The
+#      operands the block hands to the recurrence are observed through a stand-in for oracle.wkv7.wkv7_base, and
+#      the expected values are formed independently with torch.nn.functional in float64.
+class Spy:
+    def __init__(self, monkeypatch, zero_out=False):
+        self.calls = []
+        real = om.o7.wkv7_base
+
+        def fake(r, w, k, v, a, b, s, length, new_starts, compat=True):
+            self.calls.append(dict(r=r[0], w=w[0], k=k[0], v=v[0], a=a[0], b=b[0]))
+            s_new, out = real(r, w, k, v, a, b, s, length, new_starts, compat=compat)
+            return s_new, (np.zeros_like(out) if zero_out else out)
+        monkeypatch.setattr(om.o7, "wkv7_base", fake)
+
+
+def att_of(model, layer):
+    return om._layer(model["blocks"], layer)["att"]
+
+
+def time_mix(model, layer, x, v_first, T, att=None):
+    att = att or att_of(model, layer)
+    L, H, S = model["blocks"]["att"]["r_k"].shape
+    state = np.zeros((1 + S, x.shape[1]))
+    return om.time_mixing_seq(x, state, v_first, att, T, np.zeros(T, bool), H, S, layer)
+
+
+def tt(x):
+    return torch.from_numpy(np.ascontiguousarray(x))
+
+
+def test_decay_argument_is_bounded_and_reduces_to_w0(model, monkeypatch):
+    spy = Spy(monkeypatch)
+    T, C = 9, 128
+    x = np.random.default_rng(5).standard_normal((T, C))
+    time_mix(model, 1, x, x, T)
+    w = spy.calls[-1]["w"].reshape(T, C)
+    assert np.all(w <= -0.5)                                   # rwkv7.py:236: -softplus(.) - 0.5
+    att = dict(att_of(model, 1))
+    att["w1"] = np.zeros_like(att["w1"])
+    time_mix(model, 1, x, x, T, att)
+    expect = -0.5 - torch.nn.functional.softplus(-tt(att["w0"])).numpy()
+    np.testing.assert_allclose(spy.calls[-1]["w"].reshape(T, C), np.broadcast_to(expect, (T, C)), rtol=1e-12)
+
+
+def test_key_scaling_removal_vector_and_its_gate(model, monkeypatch):
+    spy = Spy(monkeypatch)
+    T, C = 7, 128
+    x = np.random.default_rng(6).standard_normal((T, C))
+    att = dict(att_of(model, 0))
+    att["x_k"] = np.zeros_like(att["x_k"])                     # no token shift in the key path: xk = x
+    k_plain = (tt(x) @ tt(att["key"]["weight"]).T).numpy()
+    # a == 1 (a0 -> +inf, no LoRA): k' = k ; the removal vector is -normalize(k k_k) per head, b = kk a = kk
+    a1 = dict(att)
+    a1["a0"] = np.full_like(att["a0"], 50.0)
+    a1["a1"] = np.zeros_like(att["a1"])
+    time_mix(model, 0, x, x, T, a1)
+    c = spy.calls[-1]
+    np.testing.assert_allclose(c["k"].reshape(T, C), k_plain, rtol=1e-10, atol=1e-12)
+    kk = torch.nn.functional.normalize((tt(k_plain) * tt(att["k_k"])).reshape(T, 2, 64), dim=-1).numpy()
+    np.testing.assert_allclose(c["a"], -kk, rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(c["b"], kk, rtol=1e-10, atol=1e-12)
+    # k_a == 0: k' = k whatever a is; b = kk sigmoid(a0 + ...)
+    a2 = dict(att)
+    a2["k_a"] = np.zeros_like(att["k_a"])
+    a2["a1"] = np.zeros_like(att["a1"])
+    time_mix(model, 0, x, x, T, a2)
+    c = spy.calls[-1]
+    np.testing.assert_allclose(c["k"].reshape(T, C), k_plain, rtol=1e-10, atol=1e-12)
+    gate = torch.sigmoid(tt(att["a0"])).numpy().reshape(2, 64)
+    np.testing.assert_allclose(c["b"], kk * gate, rtol=1e-10, atol=1e-12)
+    # general a, k_a: k' = k (1 + (a - 1) k_a)
+    a3 = dict(att)
+    a3["a1"] = np.zeros_like(att["a1"])
+    time_mix(model, 0, x, x, T, a3)
+    expect = k_plain * (1 + (torch.sigmoid(tt(att["a0"])).numpy() - 1) * att["k_a"])
+    np.testing.assert_allclose(spy.calls[-1]["k"].reshape(T, C), expect, rtol=1e-10, atol=1e-12)
+
+
+def test_value_residual_mix(model, monkeypatch):
+    spy = Spy(monkeypatch)
+    T, C = 6, 128
+    g = np.random.default_rng(7)
+    x, vf = g.standard_normal((T, C)), g.standard_normal((T, C))
+    att0 = dict(att_of(model, 0))
+    att0["x_v"] = np.zeros_like(att0["x_v"])
+    v_plain = (tt(x) @ tt(att0["value"]["weight"]).T).numpy()
+    _, _, v_first = time_mix(model, 0, x, vf, T, att0)        # layer 0: v_first is this layer's v
+    np.testing.assert_allclose(v_first, v_plain, rtol=1e-10, atol=1e-12)
+    np.testing.assert_allclose(spy.calls[-1]["v"].reshape(T, C), v_plain, rtol=1e-10, atol=1e-12)
+    att1 = dict(att_of(model, 1))
+    att1["v1"] = np.zeros_like(att1["v1"])
+    att1["v0"] = np.full_like(att1["v0"], 50.0)                # gate -> 1: v = v_first
+    _, _, v_out = time_mix(model, 1, x, vf, T, att1)
+    np.testing.assert_allclose(spy.calls[-1]["v"].reshape(T, C), vf, rtol=1e-10, atol=1e-10)
+    np.testing.assert_allclose(v_out, vf)                      # passed on unchanged
+    att1["v0"] = np.full_like(att1["v0"], -50.0)               # gate -> 0: v = this layer's own projection
+    att1["x_v"] = np.zeros_like(att1["x_v"])
+    time_mix(model, 1, x, vf, T, att1)
+    own = (tt(x) @ tt(att1["value"]["weight"]).T).numpy()
+    np.testing.assert_allclose(spy.calls[-1]["v"].reshape(T, C), own, rtol=1e-10, atol=1e-10)
+
+
+def test_gate_bonus_and_output_projection(model, monkeypatch):
+    T, C = 5, 128
+    x = np.random.default_rng(8).standard_normal((T, C))
+    att = dict(att_of(model, 1))
+    g0 = dict(att)
+    g0["g2"] = np.zeros_like(att["g2"])                        # gate == 0: the block contributes nothing
+    out, _, _ = time_mix(model, 1, x, x, T, g0)
+    assert np.all(out == 0.0)
+    # recurrence output replaced by zeros: group norm gives its bias; what is left is (bias + bonus) g Wo^T
+    spy = Spy(monkeypatch, zero_out=True)
+    att["ln_x"] = {"weight": att["ln_x"]["weight"], "bias": np.random.default_rng(9).standard_normal(C)}
+    out, _, _ = time_mix(model, 1, x, x, T, att)
+    c = spy.calls[-1]
+    xg = tt(x + (np.concatenate([np.zeros((1, C)), x[:-1]]) - x) * att["x_g"])
+    gate = (torch.sigmoid(xg @ tt(att["g1"])) @ tt(att["g2"])).numpy()
+    bonus = ((tt(c["r"]) * tt(c["k"]) * tt(att["r_k"])).sum(-1, keepdim=True) * tt(c["v"])).numpy().reshape(T, C)
+    expect = ((att["ln_x"]["bias"] + bonus) * gate) @ att["output"]["weight"].T
+    np.testing.assert_allclose(out, expect, rtol=1e-9, atol=1e-12)
+    nob = dict(att)
+    nob["r_k"] = np.zeros_like(att["r_k"])                     # r_k == 0: no bonus
+    out, _, _ = time_mix(model, 1, x, x, T, nob)
+    np.testing.assert_allclose(out, (att["ln_x"]["bias"] * gate) @ att["output"]["weight"].T, rtol=1e-9, atol=1e-12)
+
+
+def test_channel_mix_without_token_shift_is_a_relu_squared_mlp(model):
+    T, C = 8, 128
+    x = np.random.default_rng(10).standard_normal((T, C))
+    ffn = dict(om._layer(model["blocks"], 0)["ffn"])
+    ffn["x_k"] = np.zeros_like(ffn["x_k"])
+    out, last = om.channel_mixing_seq(x, np.zeros((1, C)), ffn, 5, np.zeros(T, bool))
+    F = torch.nn.functional
+    ref = F.linear(F.relu(F.linear(tt(x), tt(ffn["key"]["weight"]))) ** 2, tt(ffn["value"]["weight"])).numpy()
+    np.testing.assert_allclose(out, ref, rtol=1e-10, atol=1e-12)
+    np.testing.assert_array_equal(last, x[4])
+    # with the shift: xk = x + (prev - x) x_k, prev = state row for t = 0 and zero at a reset
+    ffn = om._layer(model["blocks"], 0)["ffn"]
+    ns = np.zeros(T, bool)
+    ns[3] = True
+    st = np.random.default_rng(11).standard_normal((1, C))
+    out, _ = om.channel_mixing_seq(x, st, ffn, T, ns)
+    prev = np.concatenate([st, x[:-1]])
+    prev[3] = 0.0
+    xk = tt(x + (prev - x) * ffn["x_k"])
+    ref = F.linear(F.relu(F.linear(xk, tt(ffn["key"]["weight"]))) ** 2, tt(ffn["value"]["weight"])).numpy()
+    np.testing.assert_allclose(out, ref, rtol=1e-10, atol=1e-12)
