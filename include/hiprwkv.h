@@ -144,6 +144,21 @@ int hiprwkv_wkv4_bwd(hiprwkv_stream stream, int io_dtype,
                      float* gw, float* gu, void* gk, void* gv, void* gs,
                      void* workspace, size_t workspace_bytes, unsigned flags);
 
+/* hiprwkv_wkv4_bwd for callers that cannot allocate device memory (code under HIP graph capture, serving loops,
+ * harnesses that forbid hipMalloc): the same kernels, with the checkpoint workspace in a 16 MiB array that is part
+ * of the library's device image (one copy per GPU, held until the process ends) instead of a caller's buffer.  It has
+ * no counterpart in the reference.  Calls nothing that allocates.  Shapes whose checkpoints
+ * (hiprwkv_wkv4_bwd_workspace_bytes) exceed hiprwkv_wkv4_bwd_noalloc_max_bytes() are refused with HIPRWKV_ENOSPACE.
+ * Every call on a GPU shares that GPU's array: calls that overlap in time on one GPU (different streams) race; calls
+ * on one stream, or ordered by events, do not.  Nothing in the array needs clearing between calls (each call writes
+ * every checkpoint before it reads it). */
+size_t hiprwkv_wkv4_bwd_noalloc_max_bytes(void);
+int hiprwkv_wkv4_bwd_noalloc(hiprwkv_stream stream, int io_dtype,
+                             int64_t B, int64_t T, int64_t C,
+                             const void* w, const void* u, const void* k, const void* v, const void* gy, const void* s,
+                             const uint32_t* length, const uint8_t* new_starts, const void* gs_new,
+                             float* gw, float* gu, void* gk, void* gv, void* gs, unsigned flags);
+
 /* ---- RWKV-7 time-mixing stages around the op (forward only) -------------------------
  * The element-wise work the reference does in jnp on either side of inner_loop (rwkv7.py:248-252, 257 and :263-265),
  * fused into one pass each; it has no counterpart among the reference's ffi targets.  `rows` = number of tokens

@@ -33,6 +33,8 @@ SIGNATURES = {
     "hiprwkv_wkv4_bwd_workspace_bytes": (_sz, [_i64] * 3),
     "hiprwkv_wkv4_bwd": (_int, [_vp, _int, _i64, _i64, _i64] + [_vp] * 6 + [_vp, _vp] + [_vp] + [_vp] * 5
                          + [_vp, _sz, _u32]),
+    "hiprwkv_wkv4_bwd_noalloc_max_bytes": (_sz, []),
+    "hiprwkv_wkv4_bwd_noalloc": (_int, [_vp, _int, _i64, _i64, _i64] + [_vp] * 6 + [_vp, _vp] + [_vp] + [_vp] * 5 + [_u32]),
     "hiprwkv_rwkv7_premix": (_int, [_vp, _int, _i64, _i64, _i64] + [_vp] * 7),
     "hiprwkv_rwkv7_postmix": (_int, [_vp, _int, _i64, _i64, _i64] + [_vp] * 8 + [ctypes.c_float, _vp]),
 }

@@ -45,6 +45,35 @@ constexpr int MAX_DEVICES = 64;
 std::mutex g_sym_mu;
 unsigned* g_status_ptr[MAX_DEVICES] = {};
 
+// Workspace of hiprwkv_wkv4_bwd_noalloc: the checkpoint array of the WKV4 backward pass, (B, ceil(T/16), 3, C) fp32,
+// for callers that cannot allocate.  Every GPU the library runs on holds its own 16 MiB copy until the process
+// ends.  Host code never uses the array's name as an address: the device address is looked up once per device
+// (scratch_base) and passed to the kernels like a caller's workspace.
+constexpr size_t SCRATCH_BYTES = (size_t)16 << 20;
+static __device__ __align__(256) __attribute__((used)) unsigned char scratch[SCRATCH_BYTES];
+void* g_scratch_ptr[MAX_DEVICES] = {};
+
+// Device address of the current device's scratch array; null (with the error text set) when the lookup fails.
+void* scratch_base() {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+    fail(HIPRWKV_ELAUNCH, "wkv4_bwd_noalloc: no usable current device (%s)", hipGetErrorString(e));
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_sym_mu);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) {
+      fail(HIPRWKV_ELAUNCH, "wkv4_bwd_noalloc: hipGetSymbolAddress failed (%s)", hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = p;
+  }
+  return g_scratch_ptr[dev];
+}
+
 // Address of the current device's failure counter, or null when it cannot be obtained (the kernels then skip the
 // count; the NaN poisoning does not depend on it).
 unsigned* status_word() {
@@ -287,6 +316,24 @@ int hiprwkv_wkv4_bwd(hiprwkv_stream stream, int io_dtype, int64_t B, int64_t T, 
   hipError_t e = launch_wkv4_bwd(A, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "wkv4_bwd: %s", hipGetErrorString(e));
   return HIPRWKV_OK;
+}
+
+size_t hiprwkv_wkv4_bwd_noalloc_max_bytes(void) { return SCRATCH_BYTES; }
+
+int hiprwkv_wkv4_bwd_noalloc(hiprwkv_stream stream, int io_dtype, int64_t B, int64_t T, int64_t C, const void* w,
+                             const void* u, const void* k, const void* v, const void* gy, const void* s,
+                             const uint32_t* length, const uint8_t* new_starts, const void* gs_new, float* gw,
+                             float* gu, void* gk, void* gv, void* gs, unsigned flags) {
+  if (B <= 0 || T <= 0 || C <= 0) return fail(HIPRWKV_EINVAL, "wkv4_bwd_noalloc: B,T,C must be positive");
+  const size_t need = hiprwkv_wkv4_bwd_workspace_bytes(B, T, C);
+  if (need > SCRATCH_BYTES)
+    return fail(HIPRWKV_ENOSPACE,
+                "wkv4_bwd_noalloc: B*ceil(T/16)*3*C*4 = %zu bytes of checkpoints exceed the built-in %zu-byte "
+                "scratch; use hiprwkv_wkv4_bwd with a caller-provided workspace", need, SCRATCH_BYTES);
+  void* ws = scratch_base();
+  if (ws == nullptr) return HIPRWKV_ELAUNCH;
+  return hiprwkv_wkv4_bwd(stream, io_dtype, B, T, C, w, u, k, v, gy, s, length, new_starts, gs_new, gw, gu, gk, gv,
+                          gs, ws, SCRATCH_BYTES, flags);
 }
 
 int hiprwkv_rwkv7_premix(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t H, int64_t N, const void* k,
