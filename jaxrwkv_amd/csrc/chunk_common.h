@@ -25,9 +25,10 @@ constexpr float MIN_CUM_L2 = -80.0f * LOG2E;    // floor of a chunk's total log2
 // a waiter that gives up sets `broken` and returns false, its wave leaves its chunk loop, and after the
 // workgroup's final barrier every output of that (sequence, head) is overwritten with NaN and the library's
 // failure counter is incremented (finish_head below), so no launch returns stale data unnoticed.
+constexpr int MAX_RING = 16;      // most slots a ring may have
 struct __attribute__((aligned(16))) Sync {
-  int ready[8];
-  int consumed[NCONS][8];
+  int ready[MAX_RING];
+  int consumed[NCONS][MAX_RING];
   int broken;
   int pad[3];
 };
@@ -49,6 +50,31 @@ __device__ __forceinline__ bool wait_consumed(Sync* sy, int slot, int want, int 
   }
   __hip_atomic_store(&sy->broken, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   return false;
+}
+
+// The same two waits for kernels whose producers run far ahead of the consumers.  A producer that finds its slot
+// still in use sleeps for hundreds of cycles between polls (every poll costs vector instructions that compete with
+// the consumer on the same SIMD); a consumer tests a flag value that it requested earlier in the chunk, so that the
+// LDS round trip is off its critical path, and only polls if that value was not the wanted one yet.
+__device__ __forceinline__ bool wait_consumed_lazy(Sync* sy, int slot, int want, int lane) {
+  for (int spin = 0; spin < SPIN_LIMIT / 8; ++spin) {
+    int seen = want;
+    if (lane < NCONS) seen = __hip_atomic_load(&sy->consumed[lane][slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (__ballot(seen < want) == 0ull) return true;
+    __builtin_amdgcn_s_sleep(8);
+  }
+  __hip_atomic_store(&sy->broken, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  return false;
+}
+__device__ __forceinline__ int peek_ready(const Sync* sy, int slot) {
+  return __hip_atomic_load(&sy->ready[slot], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+}
+__device__ __forceinline__ bool wait_ready_peeked(Sync* sy, int slot, int want, int peeked) {
+  if (__builtin_amdgcn_readfirstlane(peeked) == want) {
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+    return true;
+  }
+  return wait_ready(sy, slot, want);
 }
 
 // Test hook (HIPRWKV_DEBUG_DROP_PUBLISH): the producer of the last step does not publish it, so that the consumers'
@@ -146,10 +172,9 @@ __device__ __forceinline__ float row_scan(float x) {
 // factor so that the total becomes MIN_CUM_L2: 1/E stays finite in fp32 and the relative weights inside the chunk
 // keep their order, at the price of an inexact (weaker) decay for that channel in that chunk.
 __device__ __forceinline__ void cap_chunk_decay(float (&E)[8], int lane) {
-  bool over = false;
-#pragma unroll
-  for (int e = 0; e < 8; ++e) over = over || (E[e] < MIN_CUM_L2);
-  if (__ballot(over) != 0ull) {
+  // one comparison of the smallest of the eight sums instead of eight
+  const float lo = fminf(fminf(fminf(E[0], E[1]), fminf(E[2], E[3])), fminf(fminf(E[4], E[5]), fminf(E[6], E[7])));
+  if (__ballot(lo < MIN_CUM_L2) != 0ull) {
     rare_path();
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
