@@ -132,9 +132,7 @@ int hiprwkv_wkv7_fwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64
   const bool small_t = T <= HIPRWKV_SMALL_T && !(flags & HIPRWKV_NO_SMALL_T);
   const bool chunked = io_dtype == HIPRWKV_BF16 && !(flags & HIPRWKV_FORCE_SEQ);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  hipError_t e = small_t ? launch_wkv7_small_t_fwd(A, st)
-                 : chunked ? ((flags & 0x200u) ? launch_wkv7_chunk_fwd_pairs(A, st) : launch_wkv7_chunk_fwd(A, st))
-                           : launch_wkv7_seq_fwd(A, st);
+  hipError_t e = small_t ? launch_wkv7_small_t_fwd(A, st) : chunked ? launch_wkv7_chunk_fwd(A, st) : launch_wkv7_seq_fwd(A, st);
   if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "wkv7_fwd: %s", hipGetErrorString(e));
   return HIPRWKV_OK;
 }

@@ -762,8 +762,6 @@ static hipError_t launch_chunk(const Wkv7Args& A, hipStream_t stream) {
   return hipGetLastError();
 }
 
-// the forward pass with bf16 hi/lo pairs in every product (kept as a cross-check of wkv7_fwd.hip)
-hipError_t launch_wkv7_chunk_fwd_pairs(const Wkv7Args& A, hipStream_t stream) { return launch_chunk<false>(A, stream); }
 
 // Reverse sweep of the backward pass: gv, the workspace dsa (cotangent of sa per token) and gs.
 hipError_t launch_wkv7_chunk_bwd_a(const Wkv7Args& A, hipStream_t stream) { return launch_chunk<true>(A, stream); }

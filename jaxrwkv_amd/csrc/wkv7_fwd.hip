@@ -36,14 +36,8 @@ namespace {
 
 using namespace chunk;
 
-#ifndef WKV7_NPROD
-#define WKV7_NPROD 8
-#endif
-#ifndef WKV7_RING
-#define WKV7_RING 10
-#endif
-constexpr int NPROD = WKV7_NPROD;   // producer waves; producer p owns chunks p, p + NPROD, ...
-constexpr int RING = WKV7_RING;     // slots in flight
+constexpr int NPROD = 8;          // producer waves; producer p owns chunks p, p + NPROD, ...
+constexpr int RING = 10;          // slots in flight
 
 typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x4_t __attribute__((ext_vector_type(4)));
@@ -554,7 +548,6 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_fwd_kernel(Wkv7Args
   if (threadIdx.x < sizeof(Sync) / sizeof(int)) reinterpret_cast<int*>(sy)[threadIdx.x] = 0;
   __syncthreads();
 
-#ifndef WKV7_UNPAIRED
   // Waves go to the four SIMDs round-robin.  Consumers are waves 0, 1, 4, 5: two of them (two independent dependency
   // chains) and one producer share each of SIMDs 0 and 1, three producers each of SIMDs 2 and 3.  Measured 3.5 %
   // faster than one consumer and two producers on every SIMD: a producer's vector instructions delay the consumer
@@ -563,10 +556,6 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_fwd_kernel(Wkv7Args
   const bool is_cons = (wave & 2) == 0 && wave < 8;
   const int cq = (wave & 1) | ((wave >> 1) & 2);                                 // waves 0,1,4,5 -> 0..3
   const int pp = wave >= 8 ? wave - 4 : ((wave & 1) | ((wave >> 1) & 2));        // waves 2,3,6,7 -> 0..3, 8..11 -> 4..7
-#else
-  const bool is_cons = wave < NCONS;
-  const int cq = wave, pp = wave - NCONS;
-#endif
   if (is_cons) {
     // the chunk-to-chunk dependency runs through the consumers: let them issue ahead of the producers
     __builtin_amdgcn_s_setprio(3);
@@ -595,88 +584,35 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_fwd_kernel(Wkv7Args
       ok = wait_ready(sy, 0, 1);
       load_ops(ops, &slots[0], cq, lane);
     }
-#ifdef WKV7_PROBE
-    long long t_wait = 0, t_begin = clock64();
-#endif
     for (int j = 0; j < nch && ok; ++j) {
       const int nvalid = (j + 1 < nch || A.T % CK == 0) ? CK : (int)(A.T % CK);
       const int si = j % RING, sn = (j + 1) % RING;
       const Slot* next = (j + 1 < nch) ? &slots[sn] : nullptr;
-#ifdef WKV7_X2   // timing experiment: consumers release without consuming
-      ok = (next == nullptr) || wait_ready(sy, sn, j + 2);
-      if (false)
-#endif
       ok = consume(C, ops, &slots[si], next, snapslot, A, b, h, nvalid, j == csnap, q2drop, oc,
                    [&]() { return peek_ready(sy, sn); },
                    [&](int peeked) {
-#ifdef WKV7_PROBE
-                     const long long t0 = clock64();
-                     const bool r = wait_ready_peeked(sy, sn, j + 2, peeked);
-                     const long long t1 = clock64();
-                     t_wait += t1 - t0;
-                     if (blockIdx.x == 0 && lane == 0 && wave == 0 && A.sa != nullptr) {
-                       long long* tl = reinterpret_cast<long long*>(A.sa) + 64 + 8 * (j + 1);
-                       tl[0] = t0; tl[1] = t1;
-                     }
-                     return r;
-#else
                      return wait_ready_peeked(sy, sn, j + 2, peeked);
-#endif
                    });
       // every LDS read of slot si has returned: its data went into the MFMAs above
       if (lane == 0) __hip_atomic_store(&sy->consumed[cq][si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
-#ifdef WKV7_PROBE
-    if (blockIdx.x == 0 && lane == 0 && A.sa != nullptr) {
-      reinterpret_cast<long long*>(A.sa)[2 * wave] = clock64() - t_begin;
-      reinterpret_cast<long long*>(A.sa)[2 * wave + 1] = t_wait;
-    }
-#endif
   } else {
     const int p = pp;
     Raw raw;
     if (p < nch) load_raw(raw, A, b, h, (int64_t)p * CK, lane);
-#ifdef WKV7_PROBE
-    long long t_wait = 0, t_begin = clock64();
-#endif
     for (int j = p; j < nch; j += NPROD) {
       const int64_t c0 = (int64_t)j * CK;
       const ChunkFlags F = chunk_flags(A.ns, A.flags, A.T, b, c0, L, lane);
       const int si = j % RING;
       Slot* slot = &slots[si];
-#ifdef WKV7_PROBE
-      const long long t0 = clock64();
-      const bool okw = j < RING || wait_consumed_lazy(sy, si, j - RING + 1, lane);
-      const long long t1 = clock64();
-      t_wait += t1 - t0;
-      if (blockIdx.x == 0 && lane == 0 && A.sa != nullptr) {
-        long long* tl = reinterpret_cast<long long*>(A.sa) + 64 + 8 * j;
-        tl[2] = t0; tl[3] = t1;
-      }
-      if (!okw) break;
-#else
       if (j >= RING && !wait_consumed_lazy(sy, si, j - RING + 1, lane)) break;
-#endif
-#ifdef WKV7_X1   // timing experiment: producers publish without producing
-      if (lane == 0) { slot->keep_end = 1; slot->snap = -1; slot->keep_snap = 0; }
-#else
       mask_raw(raw, F.nvalid, lane);
       produce(lane, raw, F, slot, snapslot);
       if (j + NPROD < nch) load_raw(raw, A, b, h, c0 + (int64_t)NPROD * CK, lane);
-#endif
       if ((A.flags & FLAG_DROP_PUBLISH) && j + 1 == nch) break;
       // the release orders this wave's LDS writes before the sequence number
       if (lane == 0) __hip_atomic_store(&sy->ready[si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
-#ifdef WKV7_PROBE
-      if (blockIdx.x == 0 && lane == 0 && A.sa != nullptr) reinterpret_cast<long long*>(A.sa)[64 + 8 * j + 4] = clock64();
-#endif
     }
-#ifdef WKV7_PROBE
-    if (blockIdx.x == 0 && lane == 0 && A.sa != nullptr) {
-      reinterpret_cast<long long*>(A.sa)[2 * wave] = clock64() - t_begin;
-      reinterpret_cast<long long*>(A.sa)[2 * wave + 1] = t_wait;
-    }
-#endif
   }
   __syncthreads();
   if (head_broken(sy, A.status)) {

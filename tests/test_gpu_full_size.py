@@ -37,8 +37,10 @@ def test_wkv7_forward_and_backward_chunked_equals_sequential_at_the_headline_sha
         out[fs] = (new_s, y, sa) + tuple(g)
     torch.cuda.synchronize()
     names = ("new_s", "y", "sa", "gr", "gw", "gk", "gv", "ga", "gb", "gs")
-    # bf16 outputs differ by their rounding (rel-rms 2^-9 ~ 2e-3 each side); fp32 ones by the hi+lo operand precision
-    tol = dict(new_s=2e-5, y=4e-3, sa=1e-4, gr=4e-3, gw=6e-3, gk=4e-3, gv=4e-3, ga=4e-3, gb=4e-3, gs=1e-4)
+    # bf16 outputs differ by their rounding (rel-rms 2^-9 ~ 2e-3 each side); the fp32 ones by the operand precision of
+    # the chunked kernels: fp16 in the forward pass (state 1-2e-4, sa 3e-4), bf16 hi+lo pairs in the backward sweeps;
+    # gb = G^T sa sees the forward's sa through a sum with cancellation (5e-3 on top of its rounding)
+    tol = dict(new_s=5e-4, y=4e-3, sa=1e-3, gr=4e-3, gw=6e-3, gk=4e-3, gv=4e-3, ga=4e-3, gb=1e-2, gs=1e-4)
     for n_, c, q in zip(names, out[False], out[True]):
         assert torch.isfinite(c.float()).all(), n_
         assert rel_rms(c, q) < tol[n_], (n_, rel_rms(c, q))

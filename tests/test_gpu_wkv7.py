@@ -117,9 +117,9 @@ def test_bf16_io_against_float64_oracle():
     ref_s, ref_y = o7.wkv7_base(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], x["length"], x["new_starts"], compat=True)
     new_s, y, _ = run_fwd(x, torch.bfloat16, True)
     # y is rounded to bf16 on output: half an ulp = 2^-9 relative
-    assert_close("y", y, ref_y, rtol=2.0 ** -8, atol=1e-3)
-    # fp32 state out of the chunked MFMA kernel (operands fed as bf16 hi+lo pairs, ~16 mantissa bits)
-    assert_close("new_s", new_s, ref_s, rtol=1e-4, atol=1e-4, scale_atol=True)
+    assert_close("y", y, ref_y, rtol=2.0 ** -7, atol=2e-3, scale_atol=True)
+    # fp32 state out of the chunked MFMA kernel (fp16 operands, 11 significant bits: see test_gpu_wkv7_chunked.py)
+    assert_close("new_s", new_s, ref_s, rtol=1e-3, atol=2e-3, scale_atol=True)
     # bf16 bar: TVD of projected outputs below 1e-3, against the oracle's y rounded to the same output type
     tvd = tvd_of_projected(y, bf16_round(ref_y).astype(np.float64))
     assert tvd.max() < 1e-3, tvd.max()

@@ -1,9 +1,12 @@
 """Parity of the chunked MFMA WKV7 forward (the bf16 I/O path) against the float64 oracle on bf16-rounded inputs.
 
-Tolerances: the kernel feeds fp32 quantities to the matrix cores as bf16 hi+lo pairs (about 16 mantissa bits), so
-the fp32 results it returns (final state, sa) are held to rtol 1e-4 / atol 1e-4 x rms, and y, which is rounded to
-bf16 on output, to one bf16 ulp of the oracle's value.  The bf16 bar proper (TVD of projected outputs < 1e-3) is
-checked on a longer sequence.
+Tolerances: the kernel feeds the matrix cores fp16 operands (11 significant bits; bf16 hi+lo pairs in the Gram tiles)
+and keeps the carried state in fp32, which is what the bf16 bar (TVD of projected outputs < 1e-3, checked on a longer
+sequence) needs and no more: tests/precision_model.py predicts relative rms errors of 2e-4 for y before its rounding,
+1-2e-4 for the final state and 3e-4 for sa, and the kernel measures the same.  Element-wise that is: y within one
+bf16 ulp of the oracle plus 2e-3 of its rms, the fp32 state within 1e-3 relative plus 2e-3 of its rms (half a bf16
+ulp of a typical element: the reference returns a bf16 state for bf16 inputs, rwkv7.py:346), sa within 2e-3 relative
+plus 3e-3 of its rms.  Largest values seen over these cases and the random-shape cases: 1.1e-3, 1.3e-3, 1.4e-3.
 """
 import numpy as np
 import pytest
@@ -14,9 +17,7 @@ from tests.gpu_util import assert_close, dev, host, tvd_of_projected
 from tests.inputs import bf16_round, wkv7_inputs
 
 pytestmark = pytest.mark.gpu
-# sa carries the error of the triangular inverse, whose doubling chain runs in single bf16: rel-rms ~2e-5,
-# largest element errors ~4e-4 x rms
-SA_ATOL = 1e-3
+Y_ATOL, S_RTOL, S_ATOL, SA_RTOL, SA_ATOL = 2e-3, 1e-3, 2e-3, 2e-3, 3e-3      # atol in units of the tensor's rms
 
 
 def run(x, compat, state_dtype=torch.float32, force_seq=False, want_sa=True):
@@ -32,12 +33,12 @@ def run(x, compat, state_dtype=torch.float32, force_seq=False, want_sa=True):
 def check(x, compat, new_s, y, sa):
     ref_s, ref_y, ref_sa = o7.wkv7_base(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], x["length"],
                                         x["new_starts"], compat=compat, return_sa=True)
-    assert_close("new_s", new_s, ref_s, rtol=1e-4, atol=1e-4, scale_atol=True)
+    assert_close("new_s", new_s, ref_s, rtol=S_RTOL, atol=S_ATOL, scale_atol=True)
     if sa is not None:
-        assert_close("sa", sa, ref_sa, rtol=1e-3, atol=SA_ATOL, scale_atol=True)
+        assert_close("sa", sa, ref_sa, rtol=SA_RTOL, atol=SA_ATOL, scale_atol=True)
         assert np.all(sa[x["new_starts"]] == 0.0)        # state entering a reset token is exactly zero
-    # y is bf16 on output: within one bf16 ulp (2^-7 relative) of the oracle, plus the fp32-level slack above
-    assert_close("y", y, ref_y, rtol=2.0 ** -7, atol=1e-4, scale_atol=True)
+    # y is bf16 on output: within one bf16 ulp (2^-7 relative) of the oracle, plus the operand-precision slack above
+    assert_close("y", y, ref_y, rtol=2.0 ** -7, atol=Y_ATOL, scale_atol=True)
     if compat:
         nxt = np.zeros_like(x["new_starts"])
         nxt[:, :-1] = x["new_starts"][:, 1:]
@@ -79,8 +80,8 @@ def test_bf16_state_dtype_and_no_sa():
     new_s, y, sa = run(x, True, state_dtype=torch.bfloat16, want_sa=False)
     ref_s, ref_y = o7.wkv7_base(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], x["length"], x["new_starts"], compat=True)
     assert sa is None
-    assert_close("y", y, ref_y, rtol=2.0 ** -7, atol=1e-4, scale_atol=True)
-    assert_close("new_s", new_s, ref_s, rtol=2.0 ** -7, atol=1e-4, scale_atol=True)
+    assert_close("y", y, ref_y, rtol=2.0 ** -7, atol=Y_ATOL, scale_atol=True)
+    assert_close("new_s", new_s, ref_s, rtol=2.0 ** -7, atol=S_ATOL, scale_atol=True)
 
 
 def test_matches_sequential_kernel_and_tvd_bar():
@@ -88,8 +89,8 @@ def test_matches_sequential_kernel_and_tvd_bar():
     new_s, y, sa = run(x, True)
     ref_s, ref_y = check(x, True, new_s, y, sa)
     s2, y2, sa2 = run(x, True, force_seq=True)
-    assert_close("seq-vs-chunk new_s", new_s, s2, rtol=1e-4, atol=1e-4, scale_atol=True)
-    assert_close("seq-vs-chunk sa", sa, sa2, rtol=1e-3, atol=SA_ATOL, scale_atol=True)
+    assert_close("seq-vs-chunk new_s", new_s, s2, rtol=S_RTOL, atol=S_ATOL, scale_atol=True)
+    assert_close("seq-vs-chunk sa", sa, sa2, rtol=SA_RTOL, atol=SA_ATOL, scale_atol=True)
     # the bf16 bar: total-variation distance of projected, group-normed outputs below 1e-3
     tvd = tvd_of_projected(y, bf16_round(ref_y).astype(np.float64))
     assert tvd.max() < 1e-3, tvd.max()
