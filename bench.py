@@ -25,11 +25,22 @@ import numpy as np  # noqa: E402
 
 HBM_PEAK_GBS = 8000.0
 B, T, H, N = 8, 4096, 32, 64
-# HBM bytes per forward launch of the headline workload, from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE`
-# (scaled by a 1 GiB copy; the summary with the commands is profiles/wkv7_fwd_bwd_B8_T4096_H32_bf16.md)
-WKV7_FWD_TRAFFIC_BYTES = 948.5e6
-WKV4_FWD_TRAFFIC_BYTES = 4028.7e6     # profiles/wkv4_fwd_B32_T4096_C2560_f32.md
-WKV6_FWD_TRAFFIC_BYTES = 701.6e6      # profiles/wkv6_fwd_bwd_B16_T2048_H32_bf16.md
+# HBM bytes per forward launch from `rocprofv3 --pmc FETCH_SIZE` / `WRITE_SIZE` (scaled by a 1 GiB copy; commands and
+# figures in profiles/), each with the sha1 prefix of the kernel source it was measured on: when the source has
+# changed since, `roofline.traffic` is null instead of a stale figure.
+MEASURED_TRAFFIC = {
+    "wkv7_fwd": (948.5e6, "wkv7_fwd.hip", None),
+    "wkv4_fwd": (4028.7e6, "wkv4.hip", None),
+    "wkv6_fwd": (701.6e6, "wkv6_chunk.hip", None),
+}
+
+
+def measured_traffic(name):
+    import hashlib
+    nbytes, src, sha = MEASURED_TRAFFIC[name]
+    path = os.path.join(ROOT, "jaxrwkv_amd", "csrc", src)
+    now = hashlib.sha1(open(path, "rb").read()).hexdigest()[:12]
+    return nbytes if sha == now else None
 
 
 def make_inputs(torch, seed=0):
@@ -185,8 +196,8 @@ def bench_wkv7(torch, ops, args):
     out = base_record("WKV7 fwd tokens/s (B8 T4096 H32 N64 bf16)", tokens / (ms_step * 1e-3), ms_step, args, "bf16",
                       "isolated WKV7 op, B=8 T=4096 H=32 N=64, bf16 r/w/k/v/a/b/y, fp32 state, "
                       "new_starts~Bernoulli(1/1024), length~U{T/2..T} (BASELINE configs[1])",
-                      {"kernel": "sequential fp32 VALU" if args.seq else "chunked MFMA (bf16 hi+lo operands, fp32 accumulate)"})
-    out["roofline"] = roofline(fwd_bytes, kern_ms, None if args.seq else WKV7_FWD_TRAFFIC_BYTES)
+                      {"kernel": "sequential fp32 VALU" if args.seq else "chunked MFMA (fp16 operands, bf16 pairs in the Gram tiles, fp32 state)"})
+    out["roofline"] = roofline(fwd_bytes, kern_ms, None if args.seq else measured_traffic("wkv7_fwd"))
     if not args.no_bwd:
         def fwd_bwd():
             new_s, y, sa = ops.wkv7_fwd(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], x["length"],
@@ -229,7 +240,7 @@ def bench_wkv6(torch, ops, args):
                       "isolated WKV6 op, B=16 T=2048 H=32 N=64 bf16, zero state, new_starts~Bernoulli(1/512) "
                       "(BASELINE configs[2])",
                       {"kernel": "chunked MFMA forward and backward (bf16 hi+lo operands, fp32 accumulate)"})
-    out["roofline"] = roofline(fwd_bytes, kern_ms, WKV6_FWD_TRAFFIC_BYTES)
+    out["roofline"] = roofline(fwd_bytes, kern_ms, measured_traffic("wkv6_fwd"))
     if not args.no_bwd:
         fb = lambda: ops.wkv6_bwd(r, k, v, w, u, s, None, ns, dy, None, compat=True)
         n2 = max(2, args.steps // 4)
@@ -260,7 +271,17 @@ def bench_wkv4(torch, ops, args):
     out = base_record("WKV4 fwd tokens/s (B32 T4096 C2560 fp32)", tokens / (ms_step * 1e-3), ms_step, args, "f32",
                       "isolated WKV4 op, B=32 T=4096 C=2560 fp32, state (0,0,-1e38), length~U{1024..4096} "
                       "(BASELINE configs[3])", {"kernel": "one thread per (sequence, channel)"})
-    out["roofline"] = roofline(fwd_bytes, kern_ms, WKV4_FWD_TRAFFIC_BYTES)
+    out["roofline"] = roofline(fwd_bytes, kern_ms, measured_traffic("wkv4_fwd"))
+    if not args.no_bwd:
+        gy = f(g.standard_normal((b4, t4, c4), dtype=np.float32))
+        bwd = lambda: ops.wkv4_bwd(w, u, k, v, s, length, None, gy, None, compat=True)
+        n2 = max(2, args.steps // 4)
+        wall2, kern2 = time_region(torch, bwd, n2, 1)
+        # backward alone: reads k, v, gy and writes gk, gv (fp32)
+        bwd_bytes = 5 * tokens * c4 * 4
+        out["bwd"] = {"ms_per_call": kern2, "hbm_frac": bwd_bytes / (kern2 * 1e-3) / 1e9 / HBM_PEAK_GBS,
+                      "algorithmic_bytes": bwd_bytes, "note": "checkpoint pass + reverse pass; workspace and the "
+                      "per-sequence gw/gu sums on the host are inside the figure"}
     return out
 
 
