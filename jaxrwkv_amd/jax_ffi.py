@@ -48,6 +48,11 @@ def register():
 
 
 def _call(target, result_types, *operands):
+    # vmap_method="broadcast_all" hands a vmapped call to the handler with the mapped axes as extra LEADING
+    # dimensions on every operand (unmapped operands are broadcast to the same leading shape, at the cost of a
+    # copy).  The handlers in csrc/xla_ffi.cc rely on exactly that: they take the last three (WKV4: two) dimensions
+    # as (T, H, N) and fold everything before them into one flat batch B, for the state, length and new_starts
+    # operands too.  An operand vmapped with a non-leading out-axis would break this; jax.ffi never produces one.
     return jax.ffi.ffi_call(target, result_types, vmap_method="broadcast_all")(*operands, flags=np.int64(COMPAT_ASSOC))
 
 

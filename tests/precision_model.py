@@ -1,6 +1,6 @@
 """NumPy model of the chunked WKV7 forward kernel with a selectable operand precision for every matrix product.
 
-The chunked kernel (jaxrwkv_amd/csrc/wkv7_chunk.hip) evaluates 16 tokens at a time from the entering state S0
+The chunked kernel (jaxrwkv_amd/csrc/wkv7_fwd.hip) evaluates 16 tokens at a time from the entering state S0
 (recurrence: /root/reference/src/jaxrwkv/rwkv7.py:200-220).  With l_t = log d_t, Lc_t = sum_{s<=t} l_s:
 
     at_t = a_t exp(Lc_{t-1})   qt_t = r_t exp(Lc_t)   kh_s = k_s exp(-Lc_s)   bh_s = b_s exp(-Lc_s)
