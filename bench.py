@@ -214,11 +214,33 @@ def bench_wkv7(torch, ops, args):
                           "note": "backward = three sweeps (reverse, forward, reverse), " +
                                   ("sequential fp32 VALU kernels" if args.seq else "chunked MFMA kernels") +
                                   "; dsa and the decay-gradient terms pass through an fp32 workspace"}
+    if not args.no_fp32:
+        # the same shape with fp32 r/w/k/v/a/b/y: the chunked kernel on fp32 matrix instructions (or, with --seq, the
+        # sequential kernel); 14 token tensors' worth of bytes against the same 8 TB/s
+        x32 = {n: (x[n].float() if n in "rwkvab" else x[n]) for n in x}
+
+        def fwd32():
+            return ops.wkv7_fwd(x32["r"], x32["w"], x32["k"], x32["v"], x32["a"], x32["b"], x32["s"], x32["length"],
+                                x32["new_starts"], compat=True, want_sa=False, force_seq=args.seq)
+        n3 = max(2, args.steps // 4)
+        _, k32 = time_region(torch, fwd32, n3, 2)
+        b32 = 7 * tokens * H * N * 4 + 2 * B * H * N * N * 4 + B * T + B * 4
+        out["fp32_io"] = {"tokens_per_s": tokens / (k32 * 1e-3), "kernel_ms": k32,
+                          "hbm_frac": b32 / (k32 * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": b32,
+                          "mfma_frac": None if args.seq else fp32_mfma_flops(tokens) / (k32 * 1e-3) / 1e12 / 157.3,
+                          "kernel": "sequential fp32 VALU" if args.seq else "chunked, v_mfma_f32_16x16x4_f32 (fp32 operands)"}
+        del x32
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
         out["cpu_baseline_sequential"] = cpu_baseline_sequential()
         out["gpu_over_cpu"] = out["value"] / out["cpu_baseline"]["value"]
     return out
+
+
+def fp32_mfma_flops(tokens):
+    """Matrix-instruction flops of the fp32 chunked forward: per (16-token chunk, head) the four consumers issue 80
+    and the producer 96 v_mfma_f32_16x16x4_f32 of 2*16*16*4 flops each."""
+    return tokens / 16 * H * (4 * 80 + 96) * 2 * 16 * 16 * 4
 
 
 def bench_wkv6(torch, ops, args):
@@ -370,6 +392,7 @@ def main():
     ap.add_argument("--workload", choices=("wkv7", "wkv6", "wkv4", "model7"), default="wkv7")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-bwd", action="store_true")
+    ap.add_argument("--no-fp32", action="store_true", help="WKV7: skip the fp32-I/O leg")
     ap.add_argument("--seq", action="store_true", help="WKV7: force the sequential fp32 VALU kernel")
     ap.add_argument("--no-stream-probe", action="store_true",
                     help="skip the streaming-bandwidth probe (three 1 GiB arrays) that is reported beside the roofline")

@@ -65,8 +65,8 @@ def wkv7_fwd(r, w, k, v, a, b, s, length=None, new_starts=None, compat=True, wan
              small_t=True, debug_flags=0):
     """r,w,k,v,a,b (B,T,H,N) fp32|bf16; s (B,H,N,N) fp32|bf16.  Returns (new_s, y, sa|None).
 
-    T <= 8 runs on the small-T (decode) kernel unless ``small_t=False``; otherwise bf16 I/O runs on the chunked MFMA
-    kernel and fp32 I/O on the sequential fp32 kernel; ``force_seq`` selects the sequential kernel for bf16 I/O."""
+    T <= 8 runs on the small-T (decode) kernel unless ``small_t=False``; otherwise on a chunked matrix-core kernel
+    (fp16 operands for bf16 I/O, fp32 operands for fp32 I/O); ``force_seq`` selects the sequential fp32 kernel."""
     lib = _lib.load()
     io = r.dtype
     r, w, k, v, a, b = (_dev(x, io) for x in (r, w, k, v, a, b))

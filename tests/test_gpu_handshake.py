@@ -68,3 +68,19 @@ def test_wkv6_forward_and_backward_poison_their_outputs_and_count():
     again = ops.wkv6_fwd(r, k, v, w, u, s)
     assert ops.handshake_failures() == before
     assert torch.equal(again[0], good[0]) and torch.equal(again[1], good[1])
+
+
+def test_wkv7_fp32_forward_poisons_its_outputs_and_counts():
+    from jaxrwkv_amd import _lib, ops
+    args, _, _ = inputs7(seed=2)
+    args = tuple(t.float() if isinstance(t, torch.Tensor) else t for t in args)
+    good = ops.wkv7_fwd(*args, want_sa=True)
+    before = ops.handshake_failures()
+    new_s, y, sa = ops.wkv7_fwd(*args, want_sa=True, debug_flags=_lib.DEBUG_DROP_PUBLISH)
+    assert ops.handshake_failures() - before == B * H
+    assert y.dtype == torch.float32 and all_nan(new_s) and all_nan(y) and all_nan(sa)
+    before = ops.handshake_failures()
+    again = ops.wkv7_fwd(*args, want_sa=True)
+    assert ops.handshake_failures() == before
+    for a_, b_ in zip(again, good):
+        assert torch.equal(a_, b_)

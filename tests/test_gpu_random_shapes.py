@@ -59,6 +59,25 @@ def test_wkv7(case):
 
 
 @pytest.mark.parametrize("case", CASES, ids=lambda c: "B{B}-T{T}-H{H}-p{p}-c{compat:d}-f{frac}".format(**c))
+def test_wkv7_fp32(case):
+    """fp32 I/O: the chunked kernel on fp32 matrix instructions and the sequential kernel, both at the fp32 bar
+    (rtol 1e-4, atol 1e-5), with exact zeros at the reset positions."""
+    from tests import test_gpu_wkv7 as t7
+    B, T, H, compat = case["B"], case["T"], case["H"], case["compat"]
+    x = wkv7_inputs(B, T, H, 64, seed=case["seed"], p_reset=case["p"], min_len_frac=case["frac"])
+    if case["frac"] == 0.0:
+        x["length"][0] = 0
+    ref_s, ref_y, ref_sa = o7.wkv7_base(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], x["length"],
+                                        x["new_starts"], compat=compat, return_sa=True)
+    for force_seq in (False, True):
+        new_s, y, sa = t7.run_fwd(x, torch.float32, compat, force_seq=force_seq)
+        assert_close("y", y, ref_y)
+        assert_close("new_s", new_s, ref_s)
+        assert_close("sa", sa, ref_sa)
+        assert np.all(sa[x["new_starts"]] == 0.0)
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "B{B}-T{T}-H{H}-p{p}-c{compat:d}-f{frac}".format(**c))
 def test_wkv6(case):
     B, T, H, compat = case["B"], case["T"], case["H"], case["compat"]
     x = wkv6_inputs(B, T, H, 64, seed=case["seed"], bf16=True, p_reset=case["p"])

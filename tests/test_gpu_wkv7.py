@@ -16,11 +16,12 @@ GOLD = os.path.join(os.path.dirname(__file__), "golden", "wkv7_small.npz")
 GRAD_ATOL = dict(r=1e-5, w=5e-5, k=1e-5, v=1e-5, a=1e-5, b=1e-5, s=1e-5)
 
 
-def run_fwd(x, dtype, compat, state_dtype=torch.float32):
+def run_fwd(x, dtype, compat, state_dtype=torch.float32, force_seq=False):
     from jaxrwkv_amd import ops
     t = {n: dev(x[n], dtype) for n in ("r", "w", "k", "v", "a", "b")}
     new_s, y, sa = ops.wkv7_fwd(t["r"], t["w"], t["k"], t["v"], t["a"], t["b"], dev(x["s"], state_dtype),
-                                dev(x["length"]), dev(x["new_starts"]), compat=compat, want_sa=True, small_t=False)
+                                dev(x["length"]), dev(x["new_starts"]), compat=compat, want_sa=True, small_t=False,
+                                force_seq=force_seq)
     torch.cuda.synchronize()
     return host(new_s), host(y), host(sa)
 
