@@ -159,7 +159,7 @@ int hiprwkv_wkv4_bwd_noalloc(hiprwkv_stream stream, int io_dtype,
                              const uint32_t* length, const uint8_t* new_starts, const void* gs_new,
                              float* gw, float* gu, void* gk, void* gv, void* gs, unsigned flags);
 
-/* ---- RWKV-7 time-mixing stages around the op (forward only) -------------------------
+/* ---- RWKV-7 time-mixing stages around the op ------------------------------------------
  * The element-wise work the reference does in jnp on either side of inner_loop (rwkv7.py:248-252, 257 and :263-265),
  * fused into one pass each; it has no counterpart among the reference's ffi targets.  `rows` = number of tokens
  * (all batch axes flattened), tensors (rows, H, 64) io_dtype, parameters k_k, k_a, ln_w, ln_b, r_k (H, 64) io_dtype.
@@ -171,6 +171,21 @@ int hiprwkv_rwkv7_premix(hiprwkv_stream stream, int io_dtype, int64_t rows, int6
 int hiprwkv_rwkv7_postmix(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t H, int64_t N,
                           const void* y, const void* r, const void* k, const void* v, const void* g,
                           const void* ln_w, const void* ln_b, const void* r_k, float eps, void* out);
+
+/* Their backward passes (what jax.grad derives for rwkv7.py:248-252, 257 and :263-265).  The forward quantities are
+ * recomputed from the same inputs; nothing is saved.  Cotangents of tensors are io_dtype (rows, H, 64); cotangents of
+ * the per-head parameters (sums over all rows) are always fp32 (H, 64) and are overwritten, not accumulated into.
+ *   premix_bwd : from the cotangents of k_out, a_out, b_out to those of k, a, k_k, k_a
+ *   postmix_bwd: from the cotangent of out to those of y, r, k, v, g, ln_w, ln_b, r_k */
+int hiprwkv_rwkv7_premix_bwd(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t H, int64_t N,
+                             const void* k, const void* a, const void* k_k, const void* k_a,
+                             const void* gk_out, const void* ga_out, const void* gb_out,
+                             void* gk, void* ga, float* gk_k, float* gk_a);
+int hiprwkv_rwkv7_postmix_bwd(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t H, int64_t N,
+                              const void* y, const void* r, const void* k, const void* v, const void* g,
+                              const void* ln_w, const void* ln_b, const void* r_k, float eps, const void* gout,
+                              void* gy, void* gr, void* gk, void* gv, void* gg,
+                              float* gln_w, float* gln_b, float* gr_k);
 
 #ifdef __cplusplus
 }

@@ -37,6 +37,8 @@ SIGNATURES = {
     "hiprwkv_wkv4_bwd_noalloc": (_int, [_vp, _int, _i64, _i64, _i64] + [_vp] * 6 + [_vp, _vp] + [_vp] + [_vp] * 5 + [_u32]),
     "hiprwkv_rwkv7_premix": (_int, [_vp, _int, _i64, _i64, _i64] + [_vp] * 7),
     "hiprwkv_rwkv7_postmix": (_int, [_vp, _int, _i64, _i64, _i64] + [_vp] * 8 + [ctypes.c_float, _vp]),
+    "hiprwkv_rwkv7_premix_bwd": (_int, [_vp, _int, _i64, _i64, _i64] + [_vp] * 11),
+    "hiprwkv_rwkv7_postmix_bwd": (_int, [_vp, _int, _i64, _i64, _i64] + [_vp] * 8 + [ctypes.c_float] + [_vp] * 9),
 }
 
 _lib = None

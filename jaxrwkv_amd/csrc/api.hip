@@ -93,7 +93,7 @@ unsigned* status_word() {
 extern "C" {
 
 const char* hiprwkv_last_error(void) { return g_err; }
-int hiprwkv_version(void) { return 101; }
+int hiprwkv_version(void) { return 102; }
 
 int hiprwkv_handshake_failures(hiprwkv_stream stream, unsigned* count) {
   if (count == nullptr) return fail(HIPRWKV_EINVAL, "handshake_failures: null count pointer");
@@ -368,6 +368,43 @@ int hiprwkv_rwkv7_postmix(hiprwkv_stream stream, int io_dtype, int64_t rows, int
   hipError_t e = launch_rwkv7_postmix(io_dtype == HIPRWKV_F32, rows, H, y, r, k, v, g, ln_w, ln_b, r_k, eps, out,
                                       static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "rwkv7_postmix: %s", hipGetErrorString(e));
+  return HIPRWKV_OK;
+}
+
+int hiprwkv_rwkv7_premix_bwd(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t H, int64_t N, const void* k,
+                             const void* a, const void* k_k, const void* k_a, const void* gk_out, const void* ga_out,
+                             const void* gb_out, void* gk, void* ga, float* gk_k, float* gk_a) {
+  if (!dtype_ok(io_dtype)) return fail(HIPRWKV_EINVAL, "rwkv7_premix_bwd: dtype must be HIPRWKV_F32 or HIPRWKV_BF16");
+  if (N != 64) return fail(HIPRWKV_EINVAL, "rwkv7_premix_bwd: head size N=%lld not supported (64 only)", (long long)N);
+  if (rows <= 0 || H <= 0 || H > 65536 || (rows * H + 3) / 4 > 0x7fffffffLL)
+    return fail(HIPRWKV_EINVAL, "rwkv7_premix_bwd: bad rows/H");
+  const void* req[] = {k, a, k_k, k_a, gk_out, ga_out, gb_out, gk, ga, gk_k, gk_a};
+  for (const void* p : req) {
+    if (p == nullptr) return fail(HIPRWKV_EINVAL, "rwkv7_premix_bwd: null tensor pointer");
+    if (!aligned16(p)) return fail(HIPRWKV_EINVAL, "rwkv7_premix_bwd: tensor pointers must be 16-byte aligned");
+  }
+  hipError_t e = launch_rwkv7_premix_bwd(io_dtype == HIPRWKV_F32, rows, H, k, a, k_k, k_a, gk_out, ga_out, gb_out, gk,
+                                         ga, gk_k, gk_a, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "rwkv7_premix_bwd: %s", hipGetErrorString(e));
+  return HIPRWKV_OK;
+}
+
+int hiprwkv_rwkv7_postmix_bwd(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t H, int64_t N, const void* y,
+                              const void* r, const void* k, const void* v, const void* g, const void* ln_w,
+                              const void* ln_b, const void* r_k, float eps, const void* gout, void* gy, void* gr,
+                              void* gk, void* gv, void* gg, float* gln_w, float* gln_b, float* gr_k) {
+  if (!dtype_ok(io_dtype)) return fail(HIPRWKV_EINVAL, "rwkv7_postmix_bwd: dtype must be HIPRWKV_F32 or HIPRWKV_BF16");
+  if (N != 64) return fail(HIPRWKV_EINVAL, "rwkv7_postmix_bwd: head size N=%lld not supported (64 only)", (long long)N);
+  if (rows <= 0 || H <= 0 || H > 65536 || (rows * H + 3) / 4 > 0x7fffffffLL)
+    return fail(HIPRWKV_EINVAL, "rwkv7_postmix_bwd: bad rows/H");
+  const void* req[] = {y, r, k, v, g, ln_w, ln_b, r_k, gout, gy, gr, gk, gv, gg, gln_w, gln_b, gr_k};
+  for (const void* p : req) {
+    if (p == nullptr) return fail(HIPRWKV_EINVAL, "rwkv7_postmix_bwd: null tensor pointer");
+    if (!aligned16(p)) return fail(HIPRWKV_EINVAL, "rwkv7_postmix_bwd: tensor pointers must be 16-byte aligned");
+  }
+  hipError_t e = launch_rwkv7_postmix_bwd(io_dtype == HIPRWKV_F32, rows, H, y, r, k, v, g, ln_w, ln_b, r_k, eps, gout,
+                                          gy, gr, gk, gv, gg, gln_w, gln_b, gr_k, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "rwkv7_postmix_bwd: %s", hipGetErrorString(e));
   return HIPRWKV_OK;
 }
 

@@ -101,5 +101,12 @@ hipError_t launch_rwkv7_premix(int io_f32, int64_t rows, int64_t H, const void* 
 hipError_t launch_rwkv7_postmix(int io_f32, int64_t rows, int64_t H, const void* y, const void* r, const void* k,
                                 const void* v, const void* g, const void* ln_w, const void* ln_b, const void* r_k,
                                 float eps, void* out, hipStream_t stream);
+hipError_t launch_rwkv7_premix_bwd(int io_f32, int64_t rows, int64_t H, const void* k, const void* a, const void* k_k,
+                                   const void* k_a, const void* gko, const void* gao, const void* gbo, void* gk,
+                                   void* ga, float* gk_k, float* gk_a, hipStream_t stream);
+hipError_t launch_rwkv7_postmix_bwd(int io_f32, int64_t rows, int64_t H, const void* y, const void* r, const void* k,
+                                    const void* v, const void* g, const void* ln_w, const void* ln_b, const void* r_k,
+                                    float eps, const void* go, void* gy, void* gr, void* gk, void* gv, void* gg,
+                                    float* gln_w, float* gln_b, float* gr_k, hipStream_t stream);
 
 }  // namespace hiprwkv

@@ -116,7 +116,7 @@ class RWKV7:
     """``forward`` / ``default_state`` with the reference's argument names; batched over the leading axis."""
 
     inner = HipRWKV
-    #: use the fused pre/post time-mixing kernels (ops.rwkv7_premix / rwkv7_postmix) when no gradient is recorded
+    #: use the fused pre/post time-mixing kernels (ops.rwkv7_premix / rwkv7_postmix), with or without autograd
     fuse_mix = True
 
     @classmethod
@@ -160,7 +160,7 @@ class RWKV7:
         g = torch.sigmoid(xg @ att["g1"]) @ att["g2"]
         new_shift = x[torch.arange(B, device=x.device), last_idx]
         s = wkv_state.reshape(B, H, N, N)
-        fused = cls.fuse_mix and not torch.is_grad_enabled()      # the fused stages have no backward
+        fused = cls.fuse_mix
         rh, wh, vh = (t.reshape(B, T, H, N) for t in (r, w, v))
         if fused:
             kh, ah, bh = ops.rwkv7_premix(k.reshape(B, T, H, N), a.reshape(B, T, H, N), att["k_k"], att["k_a"])

@@ -276,15 +276,11 @@ def wkv4(w_neg, u, k, v, s, length=None, new_starts=None, compat=True):
     return _Wkv4.apply(w_neg, u, k, v, s, length, new_starts, compat)
 
 
-# ----------------------------------------------------------------------------- RWKV-7 time-mixing stages (forward only)
-def rwkv7_premix(k, a, k_k, k_a):
-    """k, a (..., H, N); k_k, k_a (H, N).  Returns (k', a_i, b_i) of rwkv7.py:248-252, 257: kk = normalize_head(k k_k),
-    k' = k (1 + (a - 1) k_a), a_i = -kk, b_i = kk a.  No autograd: for inference paths."""
+# ----------------------------------------------------------------------------- RWKV-7 time-mixing stages
+def _premix_fwd(k, a, k_k, k_a):
     lib = _lib.load()
     io = k.dtype
     H, N = k.shape[-2:]
-    k, a = _dev(k, io), _dev(a, io)
-    k_k, k_a = _dev(k_k.reshape(H, N), io), _dev(k_a.reshape(H, N), io)
     rows = k.numel() // (H * N)
     k_out, a_out, b_out = (torch.empty_like(k) for _ in range(3))
     rc = lib.hiprwkv_rwkv7_premix(_stream(), _DT[io], rows, H, N, _p(k), _p(a), _p(k_k), _p(k_a), _p(k_out), _p(a_out),
@@ -293,17 +289,84 @@ def rwkv7_premix(k, a, k_k, k_a):
     return k_out, a_out, b_out
 
 
-def rwkv7_postmix(y, r, k, v, g, ln_w, ln_b, r_k, eps=64e-5):
-    """y, r, k, v, g (..., H, N); ln_w, ln_b, r_k (H, N).  Returns (group_norm_head(y) ln_w + ln_b + (r.k.r_k) v) g of
-    rwkv7.py:263-265.  No autograd: for inference paths."""
+def _postmix_fwd(y, r, k, v, g, ln_w, ln_b, r_k, eps):
     lib = _lib.load()
     io = y.dtype
     H, N = y.shape[-2:]
-    y, r, k, v, g = (_dev(x, io) for x in (y, r, k, v, g))
-    ln_w, ln_b, r_k = (_dev(x.reshape(H, N), io) for x in (ln_w, ln_b, r_k))
     rows = y.numel() // (H * N)
     out = torch.empty_like(y)
     rc = lib.hiprwkv_rwkv7_postmix(_stream(), _DT[io], rows, H, N, _p(y), _p(r), _p(k), _p(v), _p(g), _p(ln_w), _p(ln_b),
                                    _p(r_k), float(eps), _p(out))
     _lib.check(rc, "hiprwkv_rwkv7_postmix")
     return out
+
+
+class _Premix(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, k, a, k_k, k_a):
+        ctx.save_for_backward(k, a, k_k, k_a)
+        return _premix_fwd(k, a, k_k, k_a)
+
+    @staticmethod
+    def backward(ctx, gk_out, ga_out, gb_out):
+        k, a, k_k, k_a = ctx.saved_tensors
+        lib = _lib.load()
+        io = k.dtype
+        H, N = k.shape[-2:]
+        rows = k.numel() // (H * N)
+        gk_out, ga_out, gb_out = (_dev(x, io) for x in (gk_out, ga_out, gb_out))
+        gk, ga = torch.empty_like(k), torch.empty_like(a)
+        gk_k, gk_a = (torch.empty(H, N, dtype=torch.float32, device=k.device) for _ in range(2))
+        rc = lib.hiprwkv_rwkv7_premix_bwd(_stream(), _DT[io], rows, H, N, _p(k), _p(a), _p(k_k), _p(k_a), _p(gk_out),
+                                          _p(ga_out), _p(gb_out), _p(gk), _p(ga), _p(gk_k), _p(gk_a))
+        _lib.check(rc, "hiprwkv_rwkv7_premix_bwd")
+        return gk, ga, gk_k.to(io), gk_a.to(io)
+
+
+class _Postmix(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, y, r, k, v, g, ln_w, ln_b, r_k, eps):
+        ctx.save_for_backward(y, r, k, v, g, ln_w, ln_b, r_k)
+        ctx.eps = eps
+        return _postmix_fwd(y, r, k, v, g, ln_w, ln_b, r_k, eps)
+
+    @staticmethod
+    def backward(ctx, gout):
+        y, r, k, v, g, ln_w, ln_b, r_k = ctx.saved_tensors
+        lib = _lib.load()
+        io = y.dtype
+        H, N = y.shape[-2:]
+        rows = y.numel() // (H * N)
+        gout = _dev(gout, io)
+        gy, gr, gk, gv, gg = (torch.empty_like(y) for _ in range(5))
+        gw, gb, grk = (torch.empty(H, N, dtype=torch.float32, device=y.device) for _ in range(3))
+        rc = lib.hiprwkv_rwkv7_postmix_bwd(_stream(), _DT[io], rows, H, N, _p(y), _p(r), _p(k), _p(v), _p(g), _p(ln_w),
+                                           _p(ln_b), _p(r_k), float(ctx.eps), _p(gout), _p(gy), _p(gr), _p(gk), _p(gv),
+                                           _p(gg), _p(gw), _p(gb), _p(grk))
+        _lib.check(rc, "hiprwkv_rwkv7_postmix_bwd")
+        return gy, gr, gk, gv, gg, gw.to(io), gb.to(io), grk.to(io), None
+
+
+def rwkv7_premix(k, a, k_k, k_a):
+    """k, a (..., H, N); k_k, k_a (H, N) or (H*N,).  Returns (k', a_i, b_i) of rwkv7.py:248-252, 257:
+    kk = normalize_head(k k_k), k' = k (1 + (a - 1) k_a), a_i = -kk, b_i = kk a.  Differentiable in all four inputs
+    (the backward kernel recomputes kk; parameter cotangents are summed over the tokens in fp32)."""
+    io = k.dtype
+    H, N = k.shape[-2:]
+    k, a = _dev(k, io), _dev(a, io)
+    k_k2, k_a2 = _dev(k_k.reshape(H, N), io), _dev(k_a.reshape(H, N), io)
+    if torch.is_grad_enabled() and any(t.requires_grad for t in (k, a, k_k, k_a)):
+        return _Premix.apply(k, a, k_k2, k_a2)
+    return _premix_fwd(k, a, k_k2, k_a2)
+
+
+def rwkv7_postmix(y, r, k, v, g, ln_w, ln_b, r_k, eps=64e-5):
+    """y, r, k, v, g (..., H, N); ln_w, ln_b, r_k (H, N) or (H*N,).  Returns
+    (group_norm_head(y) ln_w + ln_b + (r.k.r_k) v) g of rwkv7.py:263-265.  Differentiable in all eight tensors."""
+    io = y.dtype
+    H, N = y.shape[-2:]
+    y, r, k, v, g = (_dev(x, io) for x in (y, r, k, v, g))
+    ln_w2, ln_b2, r_k2 = (_dev(x.reshape(H, N), io) for x in (ln_w, ln_b, r_k))
+    if torch.is_grad_enabled() and any(t.requires_grad for t in (y, r, k, v, g, ln_w, ln_b, r_k)):
+        return _Postmix.apply(y, r, k, v, g, ln_w2, ln_b2, r_k2, eps)
+    return _postmix_fwd(y, r, k, v, g, ln_w2, ln_b2, r_k2, eps)

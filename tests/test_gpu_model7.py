@@ -148,6 +148,102 @@ def test_model_with_and_without_fused_stages_agree():
     torch.testing.assert_close(a[1], b[1], rtol=1e-4, atol=1e-4)
 
 
+def _mix_reference(k, a, k_k, k_a, y, r, v, gate, lnw, lnb, r_k):
+    """Plain torch of rwkv7.py:248-252, 257, 263-265 in the tensors' own dtype promoted to fp32.  k' reaches the second
+    stage rounded to the I/O dtype, as it does between the two kernels (straight-through for the gradient)."""
+    f = lambda t: t.float()
+    kk = f(k) * f(k_k)
+    kk = kk / torch.clamp(torch.linalg.vector_norm(kk, dim=-1, keepdim=True), min=1e-12)
+    k2 = f(k) * (1 + (f(a) - 1) * f(k_a))
+    k2 = k2 + (k2.to(k.dtype).float() - k2).detach()
+    ai, bi = -kk, kk * f(a)
+    yf = f(y)
+    yn = (yf - yf.mean(-1, keepdim=True)) / torch.sqrt(yf.var(-1, unbiased=False, keepdim=True) + 64e-5) * f(lnw) + f(lnb)
+    out = (yn + (f(r) * k2 * f(r_k)).sum(-1, keepdim=True) * f(v)) * f(gate)
+    return k2, ai, bi, out
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows", [(2, 37), (1, 1), (3, 700)])
+def test_fused_time_mixing_stages_backward_against_torch_autograd(dtype, rows):
+    """The backward kernels of ops.rwkv7_premix / rwkv7_postmix against torch autograd of the plain fp32 formulas, on
+    the same (dtype-rounded) inputs and cotangents: tensor cotangents and the per-head parameter cotangents, which
+    are sums over all tokens."""
+    from jaxrwkv_amd import ops
+    g = torch.Generator("cuda").manual_seed(11)
+    B, T = rows
+    H, N = 3, 64
+    n = lambda *s: torch.randn(s, device="cuda", generator=g).to(dtype)
+    leaf = lambda t: t.detach().clone().requires_grad_()
+    k, y, r, v, gate = n(B, T, H, N), n(B, T, H, N), n(B, T, H, N), n(B, T, H, N), n(B, T, H, N)
+    a = torch.sigmoid(n(B, T, H, N).float()).to(dtype)
+    params = [n(H * N) for _ in range(5)]                         # k_k, k_a, ln_w, ln_b, r_k, flat like the model's
+    cot = [n(B, T, H, N) for _ in range(4)]                       # for k', a_i, b_i (through a stand-in op) and out
+    names = ["k", "a", "k_k", "k_a", "y", "r", "v", "g", "ln_w", "ln_b", "r_k"]
+
+    def loss(mixed):
+        k2, ai, bi, out = mixed
+        # k' also feeds postmix: its cotangent is the sum of both uses, as in the model
+        return sum((t.float() * c.float()).sum() for t, c in zip((k2, ai, bi, out), cot))
+
+    def shaped(p):
+        return p.reshape(H, N)
+
+    fused_in = [leaf(t) for t in (k, a, params[0], params[1], y, r, v, gate, params[2], params[3], params[4])]
+    fk, fa, fkk, fka, fy, fr, fv, fg, flw, flb, frk = fused_in
+    k2, ai, bi = ops.rwkv7_premix(fk, fa, fkk, fka)
+    out = ops.rwkv7_postmix(fy, fr, k2, fv, fg, flw, flb, frk, 64e-5)
+    loss((k2, ai, bi, out)).backward()
+
+    ref_in = [leaf(t) for t in (k, a, params[0], params[1], y, r, v, gate, params[2], params[3], params[4])]
+    rk_, ra, rkk, rka, ry, rr, rv, rg, rlw, rlb, rrk = ref_in
+    loss(_mix_reference(rk_, ra, shaped(rkk), shaped(rka), ry, rr, rv, rg, shaped(rlw), shaped(rlb), shaped(rrk))).backward()
+
+    for name, got, want in zip(names, fused_in, ref_in):
+        assert got.grad is not None and got.grad.shape == want.grad.shape and got.grad.dtype == dtype, name
+        gw, gg = want.grad.float(), got.grad.float()
+        scale = float(gw.pow(2).mean().sqrt()) + 1e-30
+        if dtype == torch.float32:
+            torch.testing.assert_close(gg, gw, rtol=1e-4, atol=2e-5 * scale, msg=lambda m: f"{name}: {m}")
+        else:
+            # outputs are rounded to bf16 (2^-9 relative); the reference differentiates through an unrounded k'
+            torch.testing.assert_close(gg, gw, rtol=2.0 ** -6, atol=2e-2 * scale, msg=lambda m: f"{name}: {m}")
+
+
+def test_model_gradients_with_and_without_fused_stages_agree():
+    """Training-style use: d(loss)/d(params) through the whole model with the fused stages' backward kernels against
+    the same model on plain torch ops around the same WKV kernels."""
+    from jaxrwkv_amd.model7 import RWKV7, randomize_weights
+    params = randomize_weights(17, 2, 128, 211, dtype=torch.float32, device="cuda", zero_init=False)
+    tok = torch.randint(0, 211, (2, 40), device="cuda", generator=torch.Generator("cuda").manual_seed(2))
+    state = RWKV7.default_state(params, 2)
+
+    def leaves(tree, prefix=""):
+        for key, val in tree.items():
+            if isinstance(val, dict):
+                yield from leaves(val, prefix + key + ".")
+            else:
+                yield prefix + key, val
+
+    def run(fuse):
+        for _, p in leaves(params):
+            p.grad = None
+            p.requires_grad_(p.is_floating_point())
+        RWKV7.fuse_mix = fuse
+        try:
+            logits, _ = RWKV7.forward(params, tok, state)
+            torch.nn.functional.cross_entropy(logits[:, :-1].reshape(-1, 211), tok[:, 1:].reshape(-1)).backward()
+        finally:
+            RWKV7.fuse_mix = True
+        return {name: p.grad.clone() for name, p in leaves(params) if p.grad is not None}
+
+    fused, plain = run(True), run(False)
+    assert fused.keys() == plain.keys() and any("k_k" in n for n in fused) and any("ln_x" in n for n in fused)
+    for name in fused:
+        scale = float(plain[name].pow(2).mean().sqrt()) + 1e-30
+        torch.testing.assert_close(fused[name], plain[name], rtol=1e-3, atol=1e-4 * scale, msg=lambda m: f"{name}: {m}")
+
+
 class _Bf16Op:
     """HipRWKV with the op's bf16 I/O inside an otherwise fp32 harness: r, w, k, v, a, b are rounded to bf16 before
     the call and y comes back in bf16, as in a bf16 model, but everything downstream of y stays fp32.  In a harness
