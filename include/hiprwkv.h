@@ -49,6 +49,10 @@ extern "C" {
  * that streams the state once and has no per-launch set-up; this flag sends them to the general kernels instead. */
 #define HIPRWKV_NO_SMALL_T 4u
 #define HIPRWKV_SMALL_T 8
+/* hiprwkv_wkv6_fwd / hiprwkv_wkv6_bwd: `w` is (H, N), one log decay per head channel shared by every token and
+ * sequence (RWKV-5, rwkv5.py:194 / rwkv5_2.py:198), instead of (B, T, H, N).  The backward still writes the decay
+ * cotangent per token, (B, T, H, N); the caller sums it over B and T. */
+#define HIPRWKV_W_PER_HEAD 0x10u
 /* Test hook for the chunked kernels' bounded hand-shake: the producer wave of the last chunk does not publish it, the
  * consumer waves' wait runs out (a few milliseconds), every wave still ends normally, the outputs of every
  * (sequence, head) are NaN and hiprwkv_handshake_failures() has advanced by B*H per kernel. */

@@ -12,6 +12,7 @@ F32, BF16 = 0, 1
 COMPAT_ASSOC = 1
 FORCE_SEQ = 2
 NO_SMALL_T = 4
+W_PER_HEAD = 0x10
 DEBUG_DROP_PUBLISH = 0x100
 
 _vp, _i64, _int, _u32, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_uint, ctypes.c_size_t

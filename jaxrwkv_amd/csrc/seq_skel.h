@@ -29,6 +29,7 @@ struct VecIn {
   const void* p;  // (B,T,H,64)
   int f32;        // element type: 1 = float, 0 = bf16
   int kind;       // VecKind
+  int per_head;   // 1: p is (H,64), the same vector for every token and sequence
 };
 struct VecOut {
   void* p;  // may be null: result discarded
@@ -85,7 +86,7 @@ __device__ __forceinline__ void seq_run(Step& st, const VecIn* in, const VecOut*
     if (mover && t < T) {
       const size_t off = (((size_t)b * T + t) * H + h) * N64 + col;
 #pragma unroll
-      for (int x = 0; x < NIN; ++x) ld8_any(in[x], off, pre[x]);
+      for (int x = 0; x < NIN; ++x) ld8_any(in[x], in[x].per_head ? (size_t)h * N64 + col : off, pre[x]);
     } else {
 #pragma unroll
       for (int x = 0; x < NIN; ++x)

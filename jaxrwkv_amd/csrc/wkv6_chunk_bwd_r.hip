@@ -70,7 +70,11 @@ __device__ __forceinline__ void load_raw(Raw& x, const Wkv6Args& A, int64_t b, i
       o[0] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(p) + off);
       o[1] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(p) + off + 64);
     };
-    ld(A.r, x.r); ld(A.k, x.k); ld(A.v, x.v); ld(A.w, x.w); ld(A.gy, x.dy);
+    ld(A.r, x.r); ld(A.k, x.k); ld(A.v, x.v); ld(A.gy, x.dy);
+    // a decay shared by all tokens (RWKV-5) is one (H,64) row per head
+    const size_t woff = (A.flags & FLAG_W_PER_HEAD) ? ((size_t)h * 64 + 8 * g) * 2 : off;
+    x.w[0] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(A.w) + woff);
+    x.w[1] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(A.w) + woff + 64);
   } else {
     const uint4 z = make_uint4(0, 0, 0, 0);
     x.r[0] = x.r[1] = x.k[0] = x.k[1] = x.v[0] = x.v[1] = x.w[0] = x.w[1] = x.dy[0] = x.dy[1] = z;

@@ -110,7 +110,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void wkv6_seq_fwd_kernel(Wkv6Args A) {
   }
   if (st.id.L == 0) st.snapshot();
   const int io = A.io_f32;
-  VecIn in[4] = {{A.r, io, VK_ID}, {A.k, io, VK_ID}, {A.v, io, VK_ID}, {A.w, io, VK_EXP}};
+  VecIn in[4] = {{A.r, io, VK_ID}, {A.k, io, VK_ID}, {A.v, io, VK_ID}, {A.w, io, VK_EXP, (int)((A.flags & FLAG_W_PER_HEAD) != 0)}};
   VecOut out[1] = {{A.out, io}};
   seq_run<4, 1, F6_CH, false>(st, in, out, st.id.b, st.id.h, A.T, A.H, A.ns ? A.ns + st.id.b * A.T : nullptr, smem);
 }
@@ -174,7 +174,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void wkv6_seq_bwd_f_kernel(Wkv6Args A)
 #pragma unroll
   for (int c = 0; c < 16; ++c) st.S[c] = ld_state6(A.s, A.st_f32, base + c);
   const int io = A.io_f32;
-  VecIn in[5] = {{A.r, io, VK_ID}, {A.k, io, VK_ID}, {A.v, io, VK_ID}, {A.w, io, VK_EXP}, {A.gy, io, VK_ID}};
+  VecIn in[5] = {{A.r, io, VK_ID}, {A.k, io, VK_ID}, {A.v, io, VK_ID}, {A.w, io, VK_EXP, (int)((A.flags & FLAG_W_PER_HEAD) != 0)}, {A.gy, io, VK_ID}};
   VecOut out[2] = {{A.gr, io}, {A.er, 1}};
   seq_run<5, 2, BF6_CH, false>(st, in, out, st.id.b, st.id.h, A.T, A.H, A.ns ? A.ns + st.id.b * A.T : nullptr, smem);
   if (st.id.q == 0) A.gu[((size_t)st.id.b * A.H + st.id.h) * N64 + st.id.line] = st.du;
@@ -250,7 +250,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void wkv6_seq_bwd_r_kernel(Wkv6Args A)
     st.uq[c] = ld_u(A, st.id.h, st.id.q * 16 + c);
   }
   const int io = A.io_f32;
-  VecIn in[6] = {{A.r, io, VK_ID}, {A.k, io, VK_ID}, {A.v, io, VK_ID}, {A.w, io, VK_EXP}, {A.gy, io, VK_ID}, {A.er, 1, VK_ID}};
+  VecIn in[6] = {{A.r, io, VK_ID}, {A.k, io, VK_ID}, {A.v, io, VK_ID}, {A.w, io, VK_EXP, (int)((A.flags & FLAG_W_PER_HEAD) != 0)}, {A.gy, io, VK_ID}, {A.er, 1, VK_ID}};
   VecOut out[3] = {{A.gk, io}, {A.gv, io}, {A.gw, io}};
   seq_run<6, 3, BR6_CH, true>(st, in, out, st.id.b, st.id.h, A.T, A.H, A.ns ? A.ns + st.id.b * A.T : nullptr, smem);
   const size_t base = (((size_t)st.id.b * A.H + st.id.h) * N64 + st.id.line) * N64 + st.id.q * 16;

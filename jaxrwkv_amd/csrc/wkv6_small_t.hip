@@ -46,7 +46,7 @@ __global__ __launch_bounds__(256) void wkv6_small_t_kernel(Wkv6Args A) {
   for (int64_t t = 0; t < A.T; ++t) {
     const size_t tel = (((size_t)b * A.T + t) * A.H + h) * 64;
     float w[16], r[16], k[16];
-    ld16<IO>(A.w, tel + c0, w);
+    ld16<IO>(A.w, ((A.flags & FLAG_W_PER_HEAD) ? (size_t)h * 64 : tel) + c0, w);
     ld16<IO>(A.k, tel + c0, k);
     ld16<IO>(A.r, tel + c0, r);
     const float vj = ld_f(reinterpret_cast<const IO*>(A.v) + tel + j);

@@ -26,6 +26,9 @@ struct Wkv7Args {
   unsigned* status;      // device word counting workgroups whose hand-shake gave up (may be null)
 };
 
+// Wkv6Args::flags bit: w is (H,64), shared by every token and sequence (HIPRWKV_W_PER_HEAD)
+constexpr unsigned FLAG_W_PER_HEAD = 0x10u;
+
 struct Wkv6Args {
   int64_t B, T, H;
   const void *r, *k, *v, *w, *u, *s;

@@ -141,7 +141,8 @@ def wkv7(r, w, k, v, a, b, s, length=None, new_starts=None, compat=True, force_s
 # ----------------------------------------------------------------------------- WKV6
 def wkv6_fwd(r, k, v, w, u, s, length=None, new_starts=None, compat=True, force_seq=False, small_t=True,
              debug_flags=0):
-    """r,k,v,w (B,T,H,N); u (H,N); s (B,H,N,N) [key, value].  Returns (new_s, y).
+    """r,k,v (B,T,H,N); w (B,T,H,N), or (H,N) for a log decay shared by all tokens (RWKV-5); u (H,N);
+    s (B,H,N,N) [key, value].  Returns (new_s, y).
 
     T <= 8 runs on the small-T (decode) kernel unless ``small_t=False``; otherwise bf16 inputs run on the chunked
     MFMA kernel unless ``force_seq`` asks for the sequential fp32 one."""
@@ -149,7 +150,8 @@ def wkv6_fwd(r, k, v, w, u, s, length=None, new_starts=None, compat=True, force_
     io = r.dtype
     B, T, H, N = r.shape
     r, k, v = (_dev(x, io) for x in (r, k, v))
-    w = _dev(w.reshape(B, T, H, N), io)
+    per_head = w.numel() == H * N and (B * T != 1 or w.dim() == 2)
+    w = _dev(w.reshape(H, N) if per_head else w.reshape(B, T, H, N), io)
     u = _dev(u.reshape(H, N), io)
     s = _dev(s)
     length, new_starts = _length_ns(length, new_starts, B, T, r.device)
@@ -157,20 +159,22 @@ def wkv6_fwd(r, k, v, w, u, s, length=None, new_starts=None, compat=True, force_
     new_s = torch.empty_like(s)
     rc = lib.hiprwkv_wkv6_fwd(_stream(), _DT[io], _DT[s.dtype], B, T, H, N, _p(r), _p(k), _p(v), _p(w), _p(u), _p(s),
                               _p(length), _p(new_starts), _p(y), _p(new_s),
-                              _flags(compat, force_seq, small_t, debug_flags))
+                              _flags(compat, force_seq, small_t, debug_flags) | (_lib.W_PER_HEAD if per_head else 0))
     _lib.check(rc, "hiprwkv_wkv6_fwd")
     return new_s, y
 
 
 def wkv6_bwd(r, k, v, w, u, s, length, new_starts, gy, gs_out=None, compat=True, force_seq=False, debug_flags=0):
-    """Cotangents (gr, gk, gv, gw, gu, gs) of ``wkv6_fwd``; gu is summed over the batch here.
+    """Cotangents (gr, gk, gv, gw, gu, gs) of ``wkv6_fwd``; gu is summed over the batch here, and so is gw over batch
+    and tokens when ``w`` is the shared (H,N) decay.
 
     bf16 inputs run on the chunked MFMA kernels unless ``force_seq`` asks for the sequential fp32 ones."""
     lib = _lib.load()
     io = r.dtype
     B, T, H, N = r.shape
     r, k, v, gy = (_dev(x, io) for x in (r, k, v, gy))
-    w = _dev(w.reshape(B, T, H, N), io)
+    per_head = w.numel() == H * N and (B * T != 1 or w.dim() == 2)
+    w = _dev(w.reshape(H, N) if per_head else w.reshape(B, T, H, N), io)
     u = _dev(u.reshape(H, N), io)
     s = _dev(s)
     gs_out = None if gs_out is None else _dev(gs_out, s.dtype)
@@ -182,8 +186,11 @@ def wkv6_bwd(r, k, v, w, u, s, length, new_starts, gy, gs_out=None, compat=True,
     ws = torch.empty(nbytes, dtype=torch.uint8, device=r.device)
     rc = lib.hiprwkv_wkv6_bwd(_stream(), _DT[io], _DT[s.dtype], B, T, H, N, _p(r), _p(k), _p(v), _p(w), _p(u), _p(s),
                               _p(length), _p(new_starts), _p(gy), _p(gs_out), _p(gr), _p(gk), _p(gv), _p(gw), _p(gu),
-                              _p(gs), _p(ws), nbytes, _flags(compat, force_seq, debug=debug_flags))
+                              _p(gs), _p(ws), nbytes,
+                              _flags(compat, force_seq, debug=debug_flags) | (_lib.W_PER_HEAD if per_head else 0))
     _lib.check(rc, "hiprwkv_wkv6_bwd")
+    if per_head:
+        gw = gw.float().sum((0, 1)).to(io)
     return gr, gk, gv, gw, gu.sum(0).to(io), gs
 
 

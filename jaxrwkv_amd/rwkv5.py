@@ -3,8 +3,9 @@
 
 RWKV-5 is the WKV6 recurrence with a decay that does not depend on the token: ``w`` is the decay itself
 (``exp(-exp(time_decay))``), one value per head ``(H,1,1)`` (rwkv5.py:194) or per head channel ``(H,N,1)``
-(rwkv5_2.py:198); ``time_first`` has the same shapes (rwkv5.py:195, rwkv5_2.py:199).  The adapter broadcasts
-``log(w)`` over the tokens and calls the WKV6 op, whose ``w`` is the log decay.  With bf16 I/O ``log(w)`` is rounded
+(rwkv5_2.py:198); ``time_first`` has the same shapes (rwkv5.py:195, rwkv5_2.py:199).  The adapter hands
+``log(w)`` as one ``(H,N)`` tensor to the WKV6 op (its ``w`` is the log decay; flag ``HIPRWKV_W_PER_HEAD``), so no
+per-token decay is materialised; the decay cotangent comes back summed over batch and tokens.  With bf16 I/O ``log(w)`` is rounded
 to bf16 once more (relative error of the decay 2^-9 |log w| per step).
 """
 import torch
@@ -24,8 +25,7 @@ class HipRWKV:
             if torch.is_tensor(new_starts) and new_starts.dim() == 1:
                 new_starts = new_starts[None]
         B, T, H, N = r.shape
-        logw = torch.log(w.float().reshape(H, -1)).expand(H, N)
-        logw = logw.to(r.dtype)[None, None].expand(B, T, H, N).contiguous()
+        logw = torch.log(w.float().reshape(H, -1)).expand(H, N).to(r.dtype).contiguous()   # HIPRWKV_W_PER_HEAD
         u = time_first.reshape(H, -1).expand(H, N).contiguous()
         new_s, y = ops.wkv6(r, k, v, logw, u, s, length, new_starts, cls.assoc_compat)
         new_s = new_s.to(r.dtype)

@@ -47,3 +47,42 @@ def test_bf16(per_channel):
     # log(w) is rounded to bf16 once more: 2^-9 |log w| per step on the decay
     assert_close("y", host(y), ref_y, rtol=2.0 ** -6, atol=2e-2, scale_atol=True)
     assert_close("new_s", host(new_s), bf16_round(ref_s).astype(np.float64), rtol=2.0 ** -6, atol=2e-2, scale_atol=True)
+
+
+@pytest.mark.parametrize("dtype,T,force_seq", [(torch.bfloat16, 100, False), (torch.float32, 50, False),
+                                               (torch.bfloat16, 40, True), (torch.bfloat16, 5, False)])
+def test_shared_decay_equals_the_broadcast_one(dtype, T, force_seq):
+    """HIPRWKV_W_PER_HEAD: an (H,N) log decay gives bit-identical outputs and cotangents to the same decay
+    materialised per token, on the chunked, sequential and small-T kernels; its own cotangent is the per-token one
+    summed over batch and tokens."""
+    from jaxrwkv_amd import ops
+    B, H, N = 2, 3, 64
+    g = torch.Generator("cuda").manual_seed(7)
+    n = lambda *s: torch.randn(s, device="cuda", generator=g)
+    r, k, v, dy = (n(B, T, H, N).to(dtype) for _ in range(4))
+    logw = (-torch.exp(n(H, N) - 1.0)).to(dtype)
+    u = (0.5 * n(H, N)).to(dtype)
+    s, ds = 0.1 * n(B, H, N, N), n(B, H, N, N)
+    ns = torch.rand((B, T), device="cuda", generator=g) < 0.05
+    length = torch.tensor([T, max(1, T // 2)], device="cuda", dtype=torch.int32)
+    wide = logw[None, None].expand(B, T, H, N).contiguous()
+    a = ops.wkv6_fwd(r, k, v, logw, u, s, length, ns, force_seq=force_seq)
+    b = ops.wkv6_fwd(r, k, v, wide, u, s, length, ns, force_seq=force_seq)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    ga = ops.wkv6_bwd(r, k, v, logw, u, s, length, ns, dy, ds, force_seq=force_seq)
+    gb = ops.wkv6_bwd(r, k, v, wide, u, s, length, ns, dy, ds, force_seq=force_seq)
+    for i in (0, 1, 2, 4, 5):
+        assert torch.equal(ga[i], gb[i]), i
+    assert ga[3].shape == (H, N)
+    torch.testing.assert_close(ga[3].float(), gb[3].float().sum((0, 1)), rtol=2.0 ** -7 if dtype == torch.bfloat16 else 1e-5,
+                               atol=1e-5)
+
+
+def test_rwkv5_plugin_gradients_reach_the_decay():
+    from jaxrwkv_amd.rwkv5 import HipRWKV
+    r, k, v, w, u, s, length, ns = inputs(2, 48, 2, 5, True, False)
+    t = [dev(x).requires_grad_() for x in (r, k, v, w, u, s)]
+    new_s, y = HipRWKV.inner_loop(*t, dev(length), dev(ns))
+    (y.sum() + new_s.sum()).backward()
+    assert t[3].grad is not None and t[3].grad.shape == t[3].shape and bool(torch.isfinite(t[3].grad).all())
+    assert float(t[3].grad.abs().max()) > 0
