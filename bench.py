@@ -304,6 +304,16 @@ def bench_wkv4(torch, ops, args):
         out["bwd"] = {"ms_per_call": kern2, "hbm_frac": bwd_bytes / (kern2 * 1e-3) / 1e9 / HBM_PEAK_GBS,
                       "algorithmic_bytes": bwd_bytes, "note": "checkpoint pass + reverse pass; workspace and the "
                       "per-sequence gw/gu sums on the host are inside the figure"}
+
+        # training step: the forward keeps the checkpoints, the backward takes them (no checkpoint pass)
+        def fwd_bwd():
+            _, _, ck = ops.wkv4_fwd(w, u, k, v, s, length, None, compat=True, want_ckpt=True)
+            return ops.wkv4_bwd(w, u, k, v, s, length, None, gy, None, compat=True, ckpt=ck)
+        _, kern3 = time_region(torch, fwd_bwd, n2, 1)
+        fb_bytes = fwd_bytes + bwd_bytes
+        out["fwd_bwd"] = {"ms_per_step": kern3, "tokens_per_s": tokens / (kern3 * 1e-3),
+                          "hbm_frac": fb_bytes / (kern3 * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": fb_bytes,
+                          "note": "forward that also writes the state entering every 16th step + reverse pass"}
     return out
 
 

@@ -53,6 +53,9 @@ extern "C" {
  * sequence (RWKV-5, rwkv5.py:194 / rwkv5_2.py:198), instead of (B, T, H, N).  The backward still writes the decay
  * cotangent per token, (B, T, H, N); the caller sums it over B and T. */
 #define HIPRWKV_W_PER_HEAD 0x10u
+/* hiprwkv_wkv4_bwd: the workspace already holds the checkpoints that hiprwkv_wkv4_fwd_ckpt wrote for the same
+ * inputs; the backward then skips its own first pass over k and v. */
+#define HIPRWKV_CKPT_READY 0x20u
 /* Test hook for the chunked kernels' bounded hand-shake: the producer wave of the last chunk does not publish it, the
  * consumer waves' wait runs out (a few milliseconds), every wave still ends normally, the outputs of every
  * (sequence, head) are NaN and hiprwkv_handshake_failures() has advanced by B*H per kernel. */
@@ -136,6 +139,15 @@ int hiprwkv_wkv4_fwd(hiprwkv_stream stream, int io_dtype,
                      void* new_s, void* out, unsigned flags);
 
 size_t hiprwkv_wkv4_bwd_workspace_bytes(int64_t B, int64_t T, int64_t C);
+
+/* hiprwkv_wkv4_fwd for a caller that will run the backward pass (the forward rule of the custom VJP, rwkv4.py:379-383):
+ * same results, and the state entering every 16th step goes to `workspace` (hiprwkv_wkv4_bwd_workspace_bytes), which
+ * hiprwkv_wkv4_bwd then takes with HIPRWKV_CKPT_READY.  Saves that pass its re-read of k and v. */
+int hiprwkv_wkv4_fwd_ckpt(hiprwkv_stream stream, int io_dtype,
+                          int64_t B, int64_t T, int64_t C,
+                          const void* w, const void* u, const void* k, const void* v, const void* s,
+                          const uint32_t* length, const uint8_t* new_starts,
+                          void* new_s, void* out, void* workspace, size_t workspace_bytes, unsigned flags);
 
 /* Replaces ffi target "wkv4-bwd-{fp32,bf16}": operands w,u,k,v,gy,s,length,new_starts,gs_new
  * -> gw (B,C), gu (B,C), gk, gv, gs  (rwkv4.py:347-349); gw and gu are per sequence in fp32 and are summed

@@ -13,6 +13,7 @@ COMPAT_ASSOC = 1
 FORCE_SEQ = 2
 NO_SMALL_T = 4
 W_PER_HEAD = 0x10
+CKPT_READY = 0x20
 DEBUG_DROP_PUBLISH = 0x100
 
 _vp, _i64, _int, _u32, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_uint, ctypes.c_size_t
@@ -31,6 +32,8 @@ SIGNATURES = {
     "hiprwkv_wkv6_bwd": (_int, [_vp, _int, _int, _i64, _i64, _i64, _i64] + [_vp] * 6 + [_vp, _vp] + [_vp, _vp]
                          + [_vp] * 6 + [_vp, _sz, _u32]),
     "hiprwkv_wkv4_fwd": (_int, [_vp, _int, _i64, _i64, _i64] + [_vp] * 5 + [_vp, _vp] + [_vp, _vp, _u32]),
+    "hiprwkv_wkv4_fwd_ckpt": (_int, [_vp, _int, _i64, _i64, _i64] + [_vp] * 5 + [_vp, _vp] + [_vp, _vp, _vp,
+                                     ctypes.c_size_t, _u32]),
     "hiprwkv_wkv4_bwd_workspace_bytes": (_sz, [_i64] * 3),
     "hiprwkv_wkv4_bwd": (_int, [_vp, _int, _i64, _i64, _i64] + [_vp] * 6 + [_vp, _vp] + [_vp] + [_vp] * 5
                          + [_vp, _sz, _u32]),

@@ -258,9 +258,33 @@ int hiprwkv_wkv6_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64
   return HIPRWKV_OK;
 }
 
+static int wkv4_fwd_impl(hiprwkv_stream stream, int io_dtype, int64_t B, int64_t T, int64_t C, const void* w,
+                         const void* u, const void* k, const void* v, const void* s, const uint32_t* length,
+                         const uint8_t* new_starts, void* new_s, void* out, float* ckpt, unsigned flags);
+
 int hiprwkv_wkv4_fwd(hiprwkv_stream stream, int io_dtype, int64_t B, int64_t T, int64_t C, const void* w,
                      const void* u, const void* k, const void* v, const void* s, const uint32_t* length,
                      const uint8_t* new_starts, void* new_s, void* out, unsigned flags) {
+  return wkv4_fwd_impl(stream, io_dtype, B, T, C, w, u, k, v, s, length, new_starts, new_s, out, nullptr, flags);
+}
+
+int hiprwkv_wkv4_fwd_ckpt(hiprwkv_stream stream, int io_dtype, int64_t B, int64_t T, int64_t C, const void* w,
+                          const void* u, const void* k, const void* v, const void* s, const uint32_t* length,
+                          const uint8_t* new_starts, void* new_s, void* out, void* workspace, size_t workspace_bytes,
+                          unsigned flags) {
+  if (workspace == nullptr || !aligned16(workspace))
+    return fail(HIPRWKV_EINVAL, "wkv4_fwd_ckpt: workspace must be a 16-byte aligned device pointer");
+  if (B <= 0 || T <= 0 || C <= 0) return fail(HIPRWKV_EINVAL, "wkv4_fwd_ckpt: B,T,C must be positive");
+  const size_t need = hiprwkv_wkv4_bwd_workspace_bytes(B, T, C);
+  if (workspace_bytes < need)
+    return fail(HIPRWKV_ENOSPACE, "wkv4_fwd_ckpt: workspace has %zu bytes, %zu needed", workspace_bytes, need);
+  return wkv4_fwd_impl(stream, io_dtype, B, T, C, w, u, k, v, s, length, new_starts, new_s, out,
+                       static_cast<float*>(workspace), flags);
+}
+
+static int wkv4_fwd_impl(hiprwkv_stream stream, int io_dtype, int64_t B, int64_t T, int64_t C, const void* w,
+                         const void* u, const void* k, const void* v, const void* s, const uint32_t* length,
+                         const uint8_t* new_starts, void* new_s, void* out, float* ckpt, unsigned flags) {
   if (!dtype_ok(io_dtype)) return fail(HIPRWKV_EINVAL, "wkv4_fwd: dtype must be HIPRWKV_F32 or HIPRWKV_BF16");
   if (B <= 0 || T <= 0 || C <= 0) return fail(HIPRWKV_EINVAL, "wkv4_fwd: B,T,C must be positive");
   if (B * ((C + 63) / 64) > 0x7fffffffLL) return fail(HIPRWKV_EINVAL, "wkv4_fwd: B*C exceeds the grid limit");
@@ -277,6 +301,7 @@ int hiprwkv_wkv4_fwd(hiprwkv_stream stream, int io_dtype, int64_t B, int64_t T, 
   A.w = w; A.u = u; A.k = k; A.v = v; A.s = s;
   A.length = length; A.ns = new_starts;
   A.new_s = new_s; A.out = out;
+  A.ckpt = ckpt;
   A.io_f32 = io_dtype == HIPRWKV_F32;
   A.flags = flags;
   hipError_t e = launch_wkv4_fwd(A, static_cast<hipStream_t>(stream));

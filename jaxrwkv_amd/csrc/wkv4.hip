@@ -22,6 +22,7 @@ namespace hiprwkv {
 
 constexpr int W4_THREADS = 64;
 constexpr int W4_TB = 8;
+constexpr int W4_SEG = 16;                // the backward pass wants the state entering every W4_SEG-th step
 constexpr float W4_RESET_PP = -1e30f;  // rwkv4.py:149-150
 
 namespace {
@@ -140,8 +141,21 @@ __global__ __launch_bounds__(W4_THREADS) void wkv4_fwd_kernel(Wkv4Args A) {
     if (t == L - 1) snapshot();
   };
   const uint64_t block_lanes = (1ull << W4_TB) - 1ull;
+  // with a checkpoint array (a forward pass whose backward will follow) the state entering every W4_SEG-th step is
+  // kept, before that step's reset: what the backward's own first pass would recompute from k and v
+  static_assert(W4_SEG % W4_TB == 0, "segments start at block starts");
+  float* ck = A.ckpt ? A.ckpt + (size_t)b * ((A.T + W4_SEG - 1) / W4_SEG) * 3 * A.C + cc : nullptr;
+  auto checkpoint = [&](int64_t t) {
+    if (ck != nullptr && t % W4_SEG == 0) {
+      const int64_t sg = t / W4_SEG;
+      ck[(sg * 3 + 0) * A.C] = aa;
+      ck[(sg * 3 + 1) * A.C] = bb;
+      ck[(sg * 3 + 2) * A.C] = pp;
+    }
+  };
   int64_t t0 = 0;
   for (; t0 + W4_TB <= A.T; t0 += W4_TB) {
+    checkpoint(t0);
     const uint64_t rmask = ns != nullptr ? (__ballot(nsb != 0) & block_lanes) : 0ull;
     fetch_flags(t0 + W4_TB);
     // descriptors of the block: offsets stay below 2 W4_TB rows whatever the sequence length
@@ -163,6 +177,7 @@ __global__ __launch_bounds__(W4_THREADS) void wkv4_fwd_kernel(Wkv4Args A) {
   }
   // the ragged end: fewer than W4_TB tokens, their operands are in the registers already
   if (t0 < A.T) {
+    checkpoint(t0);
     const int left = (int)(A.T - t0);
     const uint64_t rmask = ns != nullptr ? (__ballot(nsb != 0) & ((1ull << left) - 1ull)) : 0ull;
     const rsrc_t ry = make_rsrc(yseq + (size_t)t0 * A.C);
@@ -182,8 +197,6 @@ __global__ __launch_bounds__(W4_THREADS) void wkv4_fwd_kernel(Wkv4Args A) {
 // step; the second kernel walks the segments backwards, recomputes the W4_SEG states of a segment into registers
 // and then differentiates its steps last to first.  Both stream their operands like the forward kernel: every
 // segment issues the same sequence of requests, each for a row that is needed a fixed number of steps later.
-constexpr int W4_SEG = 16;
-
 namespace {
 
 // the flags of a segment as a uniform mask, bit x = token t0 + x (tokens beyond the sequence have none)
@@ -426,11 +439,12 @@ __global__ __launch_bounds__(W4_THREADS) void wkv4_bwd_kernel(Wkv4Args A) {
 hipError_t launch_wkv4_bwd(const Wkv4Args& A, hipStream_t stream) {
   const int64_t cblocks = (A.C + W4_THREADS - 1) / W4_THREADS;
   const dim3 grid((unsigned)(A.B * cblocks)), block(W4_THREADS);
+  const bool have_ckpt = (A.flags & FLAG_CKPT_READY) != 0;   // written by the forward pass of the same inputs
   if (A.io_f32) {
-    hipLaunchKernelGGL(wkv4_ckpt_kernel<float>, grid, block, 0, stream, A);
+    if (!have_ckpt) hipLaunchKernelGGL(wkv4_ckpt_kernel<float>, grid, block, 0, stream, A);
     hipLaunchKernelGGL(wkv4_bwd_kernel<float>, grid, block, 0, stream, A);
   } else {
-    hipLaunchKernelGGL(wkv4_ckpt_kernel<bf16_t>, grid, block, 0, stream, A);
+    if (!have_ckpt) hipLaunchKernelGGL(wkv4_ckpt_kernel<bf16_t>, grid, block, 0, stream, A);
     hipLaunchKernelGGL(wkv4_bwd_kernel<bf16_t>, grid, block, 0, stream, A);
   }
   return hipGetLastError();

@@ -48,6 +48,9 @@ struct Wkv6Args {
   unsigned* status;   // device word counting workgroups whose hand-shake gave up (may be null)
 };
 
+// Wkv4Args::flags bit: the workspace already holds the checkpoints (HIPRWKV_CKPT_READY)
+constexpr unsigned FLAG_CKPT_READY = 0x20u;
+
 struct Wkv4Args {
   int64_t B, T, C;
   const void *w, *u, *k, *v, *s;
@@ -62,7 +65,7 @@ struct Wkv4Args {
   const void* gs_new;
   void *gk, *gv, *gs;
   float *gw, *gu;   // (B,C) each
-  float* ckpt;      // workspace: (B, ceil(T/16), 3, C) states entering every 16th step
+  float* ckpt;      // workspace: (B, ceil(T/16), 3, C) states entering every 16th step (forward: optional output)
 };
 
 // Raises a kernel's dynamic-LDS limit once per kernel and device instead of at every enqueue (the attribute call

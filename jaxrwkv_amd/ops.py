@@ -220,8 +220,10 @@ def wkv6(r, k, v, w, u, s, length=None, new_starts=None, compat=True):
 
 
 # ----------------------------------------------------------------------------- WKV4
-def wkv4_fwd(w_neg, u, k, v, s, length=None, new_starts=None, compat=True):
-    """w_neg = -exp(time_decay), u (C,); k,v (B,T,C); s (B,3,C).  Returns (new_s, wkv) -- receptance not applied."""
+def wkv4_fwd(w_neg, u, k, v, s, length=None, new_starts=None, compat=True, want_ckpt=False):
+    """w_neg = -exp(time_decay), u (C,); k,v (B,T,C); s (B,3,C).  Returns (new_s, wkv) -- receptance not applied.
+    ``want_ckpt``: also return the checkpoint workspace that ``wkv4_bwd(..., ckpt=)`` takes (the state entering every
+    16th step), so that the backward pass need not recompute it."""
     lib = _lib.load()
     io = k.dtype
     k, v, s, w_neg, u = (_dev(x, io) for x in (k, v, s, w_neg, u))
@@ -230,14 +232,22 @@ def wkv4_fwd(w_neg, u, k, v, s, length=None, new_starts=None, compat=True):
     length, new_starts = _length_ns(length, new_starts, B, T, k.device)
     y = torch.empty_like(k)
     new_s = torch.empty_like(s)
+    if want_ckpt:
+        nbytes = lib.hiprwkv_wkv4_bwd_workspace_bytes(B, T, C)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=k.device)
+        rc = lib.hiprwkv_wkv4_fwd_ckpt(_stream(), _DT[io], B, T, C, _p(w_neg), _p(u), _p(k), _p(v), _p(s), _p(length),
+                                       _p(new_starts), _p(new_s), _p(y), _p(ws), nbytes, _flags(compat))
+        _lib.check(rc, "hiprwkv_wkv4_fwd_ckpt")
+        return new_s, y, ws
     rc = lib.hiprwkv_wkv4_fwd(_stream(), _DT[io], B, T, C, _p(w_neg), _p(u), _p(k), _p(v), _p(s), _p(length),
                               _p(new_starts), _p(new_s), _p(y), _flags(compat))
     _lib.check(rc, "hiprwkv_wkv4_fwd")
     return new_s, y
 
 
-def wkv4_bwd(w_neg, u, k, v, s, length, new_starts, gy, gs_new=None, compat=True):
-    """Cotangents (gw, gu, gk, gv, gs) of ``wkv4_fwd``; gw, gu are summed over the batch here (rwkv4.py:351)."""
+def wkv4_bwd(w_neg, u, k, v, s, length, new_starts, gy, gs_new=None, compat=True, ckpt=None):
+    """Cotangents (gw, gu, gk, gv, gs) of ``wkv4_fwd``; gw, gu are summed over the batch here (rwkv4.py:351).
+    ``ckpt``: the workspace ``wkv4_fwd(..., want_ckpt=True)`` returned for the same inputs."""
     lib = _lib.load()
     io = k.dtype
     k, v, s, w_neg, u, gy = (_dev(x, io) for x in (k, v, s, w_neg, u, gy))
@@ -249,10 +259,14 @@ def wkv4_bwd(w_neg, u, k, v, s, length, new_starts, gy, gs_new=None, compat=True
     gw = torch.empty((B, C), dtype=torch.float32, device=k.device)
     gu = torch.empty((B, C), dtype=torch.float32, device=k.device)
     nbytes = lib.hiprwkv_wkv4_bwd_workspace_bytes(B, T, C)
-    ws = torch.empty(nbytes, dtype=torch.uint8, device=k.device)
+    if ckpt is None:
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=k.device)
+    else:
+        ws = ckpt
+        assert ws.dtype == torch.uint8 and ws.numel() >= nbytes and ws.is_cuda
     rc = lib.hiprwkv_wkv4_bwd(_stream(), _DT[io], B, T, C, _p(w_neg), _p(u), _p(k), _p(v), _p(gy), _p(s), _p(length),
                               _p(new_starts), _p(gs_new), _p(gw), _p(gu), _p(gk), _p(gv), _p(gs), _p(ws), nbytes,
-                              _flags(compat))
+                              _flags(compat) | (0 if ckpt is None else _lib.CKPT_READY))
     _lib.check(rc, "hiprwkv_wkv4_bwd")
     return gw.sum(0).to(io), gu.sum(0).to(io), gk, gv, gs
 
@@ -262,17 +276,17 @@ class _Wkv4(torch.autograd.Function):
 
     @staticmethod
     def forward(ctx, w_neg, u, k, v, s, length, new_starts, compat):
-        new_s, y = wkv4_fwd(w_neg, u, k, v, s, length, new_starts, compat)
+        new_s, y, ckpt = wkv4_fwd(w_neg, u, k, v, s, length, new_starts, compat, want_ckpt=True)
         ctx.compat = compat
-        ctx.save_for_backward(w_neg, u, k, v, s, length, new_starts)
+        ctx.save_for_backward(w_neg, u, k, v, s, length, new_starts, ckpt)
         return new_s, y
 
     @staticmethod
     def backward(ctx, gs_new, gy):
-        w_neg, u, k, v, s, length, new_starts = ctx.saved_tensors
+        w_neg, u, k, v, s, length, new_starts, ckpt = ctx.saved_tensors
         if gy is None:
             gy = torch.zeros_like(k)
-        gw, gu, gk, gv, gs = wkv4_bwd(w_neg, u, k, v, s, length, new_starts, gy, gs_new, ctx.compat)
+        gw, gu, gk, gv, gs = wkv4_bwd(w_neg, u, k, v, s, length, new_starts, gy, gs_new, ctx.compat, ckpt=ckpt)
         return gw, gu, gk, gv, gs, None, None, None
 
 

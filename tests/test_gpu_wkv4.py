@@ -188,3 +188,23 @@ def test_bf16_backward(B, T, C, seed, compat):
     gw, gu, gk, gv, gsi = ref
     for name, g_, rf in zip(("w", "u", "k", "v", "s"), got, (gw.sum(0), gu.sum(0), gk, gv, gsi)):
         assert_close("g" + name, host(g_), rf, rtol=2.0 ** -7, atol=1e-3, scale_atol=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_forward_checkpoints_equal_the_backward_own_pass(dtype):
+    """hiprwkv_wkv4_fwd_ckpt + HIPRWKV_CKPT_READY: same outputs as the plain forward, and the backward that takes the
+    forward's checkpoints returns bit for bit what the backward with its own checkpoint pass returns (T not a
+    multiple of the 16-step segments or of the forward's 8-step blocks, resets, ragged lengths)."""
+    from jaxrwkv_amd import ops
+    for B, T, C, seed in [(2, 77, 100, 1), (1, 16, 64, 2), (3, 5, 65, 3), (2, 129, 128, 4)]:
+        x = wkv4_inputs(B, T, C, seed=seed, p_reset=0.05, default_state=False, min_len=1)
+        g = np.random.default_rng(seed)
+        gy, gs = dev(g.standard_normal(x["k"].shape), dtype), dev(g.standard_normal(x["s"].shape), dtype)
+        a = [dev(x[n], dtype) for n in ("w", "u", "k", "v", "s")] + [dev(x["length"]), dev(x["new_starts"])]
+        plain = ops.wkv4_fwd(*a)
+        new_s, y, ck = ops.wkv4_fwd(*a, want_ckpt=True)
+        assert torch.equal(new_s, plain[0]) and torch.equal(y, plain[1])
+        own = ops.wkv4_bwd(*a, gy, gs)
+        taken = ops.wkv4_bwd(*a, gy, gs, ckpt=ck)
+        for p_, q_ in zip(own, taken):
+            assert torch.equal(p_, q_), (B, T, C)
