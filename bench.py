@@ -31,7 +31,7 @@ B, T, H, N = 8, 4096, 32, 64
 MEASURED_TRAFFIC = {
     "wkv7_fwd": (948.5e6, "wkv7_fwd.hip", None),
     "wkv4_fwd": (4028.7e6, "wkv4.hip", None),
-    "wkv6_fwd": (701.6e6, "wkv6_chunk.hip", None),
+    "wkv6_fwd": (701.6e6, "wkv6_fwd.hip", None),
 }
 
 

@@ -85,9 +85,10 @@ def test_length_zero():
 def test_bf16_io_against_float64_oracle():
     x = wkv6_inputs(2, 256, 4, 64, seed=31, bf16=True, p_reset=0.01)
     ref_s, ref_y = o6.wkv6_base(x["r"], x["k"], x["v"], x["w"], x["u"], x["s"], x["length"], x["new_starts"], compat=True)
-    new_s, y = run_fwd(x, torch.bfloat16, True)        # bf16 I/O: the chunked MFMA kernel (hi+lo bf16 operands)
-    assert_close("y", y, ref_y, rtol=2.0 ** -7, atol=1e-4, scale_atol=True)
-    assert_close("new_s", new_s, ref_s, rtol=1e-4, atol=1e-4, scale_atol=True)
+    new_s, y = run_fwd(x, torch.bfloat16, True)        # bf16 I/O: the chunked MFMA kernel (fp16 operands)
+    # tolerances of tests/test_gpu_wkv6_chunked.py
+    assert_close("y", y, ref_y, rtol=2.0 ** -7, atol=2e-3, scale_atol=True)
+    assert_close("new_s", new_s, ref_s, rtol=1e-3, atol=2e-3, scale_atol=True)
 
 
 def test_plugin_class_signature_unbatched():

@@ -1,8 +1,11 @@
 """Parity of the chunked MFMA WKV6 forward (the bf16 I/O path) against the float64 oracle on bf16-rounded inputs.
 
-Tolerances: fp32 quantities reach the matrix cores as bf16 hi+lo pairs (about 16 mantissa bits), so the fp32 final
-state is held to rtol 1e-4 / atol 1e-4 x rms, and y, which is rounded to bf16 on output, to one bf16 ulp of the
-oracle's value.  The bf16 bar proper (TVD of projected outputs < 1e-3) is checked on a longer sequence.
+Tolerances.  The kernel (jaxrwkv_amd/csrc/wkv6_fwd.hip) feeds the matrix cores fp16 operands (11 significant bits:
+the state, qt, ke, v; the Gram tile as an fp16 pair, its operands as bf16 pairs), so y before its bf16 rounding and the
+fp32 state carry relative errors of a few 1e-4 of their rms.  A scan of every case of this file and of
+tests/test_gpu_random_shapes.py found, in units of the compared array's rms, at most 1.2e-3 for y beyond one bf16 ulp
+of the oracle's value and 1.3e-3 for the state beyond 1e-3 of its own magnitude; the figures below leave a factor
+1.5 on top.  The bf16 bar proper (TVD of projected outputs < 1e-3) is checked on a longer sequence.
 """
 import numpy as np
 import pytest
@@ -13,6 +16,7 @@ from tests.gpu_util import assert_close, dev, host, tvd_of_projected
 from tests.inputs import bf16_round, wkv6_inputs
 
 pytestmark = pytest.mark.gpu
+Y_ATOL, S_RTOL, S_ATOL = 2e-3, 1e-3, 2e-3      # atol in units of the reference array's rms
 
 
 def run(x, compat, state_dtype=torch.float32, force_seq=False):
@@ -27,8 +31,8 @@ def run(x, compat, state_dtype=torch.float32, force_seq=False):
 def check(x, compat, new_s, y):
     ref_s, ref_y = o6.wkv6_base(x["r"], x["k"], x["v"], x["w"], x["u"], x["s"], x["length"], x["new_starts"],
                                 compat=compat)
-    assert_close("new_s", new_s, ref_s, rtol=1e-4, atol=1e-4, scale_atol=True)
-    assert_close("y", y, ref_y, rtol=2.0 ** -7, atol=1e-4, scale_atol=True)
+    assert_close("new_s", new_s, ref_s, rtol=S_RTOL, atol=S_ATOL, scale_atol=True)
+    assert_close("y", y, ref_y, rtol=2.0 ** -7, atol=Y_ATOL, scale_atol=True)
     return ref_s, ref_y
 
 
@@ -64,8 +68,8 @@ def test_bf16_state_dtype():
     x["s"] = bf16_round(x["s"]).astype(np.float64)
     new_s, y = run(x, True, state_dtype=torch.bfloat16)
     ref_s, ref_y = o6.wkv6_base(x["r"], x["k"], x["v"], x["w"], x["u"], x["s"], x["length"], x["new_starts"], compat=True)
-    assert_close("y", y, ref_y, rtol=2.0 ** -7, atol=1e-4, scale_atol=True)
-    assert_close("new_s", new_s, ref_s, rtol=2.0 ** -7, atol=1e-4, scale_atol=True)
+    assert_close("y", y, ref_y, rtol=2.0 ** -7, atol=Y_ATOL, scale_atol=True)
+    assert_close("new_s", new_s, ref_s, rtol=2.0 ** -7, atol=S_ATOL, scale_atol=True)
 
 
 def test_matches_sequential_kernel_and_tvd_bar():
@@ -73,8 +77,8 @@ def test_matches_sequential_kernel_and_tvd_bar():
     new_s, y = run(x, True)
     ref_s, ref_y = check(x, True, new_s, y)
     s2, y2 = run(x, True, force_seq=True)
-    assert_close("seq-vs-chunk new_s", new_s, s2, rtol=1e-4, atol=1e-4, scale_atol=True)
-    assert_close("seq-vs-chunk y", y, y2, rtol=2.0 ** -7, atol=1e-4, scale_atol=True)
+    assert_close("seq-vs-chunk new_s", new_s, s2, rtol=S_RTOL, atol=S_ATOL, scale_atol=True)
+    assert_close("seq-vs-chunk y", y, y2, rtol=2.0 ** -7, atol=Y_ATOL, scale_atol=True)
     # the bf16 bar: total-variation distance of projected, group-normed outputs below 1e-3
     tvd = tvd_of_projected(y, bf16_round(ref_y).astype(np.float64))
     assert tvd.max() < 1e-3, tvd.max()
