@@ -211,7 +211,7 @@ def bench_wkv7(torch, ops, args):
         fb_bytes = 20 * tokens * H * N * 2 + 4 * B * H * N * N * 4
         out["fwd_bwd"] = {"tokens_per_s": tokens / (ms2 * 1e-3), "ms_per_step": ms2,
                           "hbm_frac": fb_bytes / (ms2 * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": fb_bytes,
-                          "note": "backward = three sweeps (reverse, forward, reverse), " +
+                          "note": "forward keeps the residual sa (fp16 beside bf16 I/O); backward = three sweeps (reverse, forward, reverse), " +
                                   ("sequential fp32 VALU kernels" if args.seq else "chunked MFMA kernels") +
                                   "; dsa and the decay-gradient terms pass through an fp32 workspace"}
     if not args.no_fp32:

@@ -76,15 +76,17 @@ int hiprwkv_handshake_failures(hiprwkv_stream stream, unsigned* count);
 /* ---- WKV7 ------------------------------------------------------------------
  * Replaces ffi target "wkv7-fwd-{fp32,bf16}": operands w,r,k,v,a,b,s,length,new_starts
  * -> out, s_restore, sa_restore, new_s  (rwkv7.py:372-375).  `w` is the raw decay
- * argument; the op applies exp(-exp(w)) (rwkv7.py:201).  `sa` (B,T,H,N) fp32 is
- * the residual S_{t-1} a_t kept for the backward pass (the reference's sa_restore);
- * pass NULL for inference.  No state checkpoints (s_restore) are needed. */
+ * argument; the op applies exp(-exp(w)) (rwkv7.py:201).  `sa` (B,T,H,N) is
+ * the residual S_{t-1} a_t kept for the backward pass (the reference's sa_restore):
+ * fp32 beside fp32 I/O, IEEE half (2 bytes per element) beside bf16 I/O; the caller hands
+ * the same buffer to hiprwkv_wkv7_bwd.  Pass NULL for inference.  No state checkpoints
+ * (s_restore) are needed. */
 int hiprwkv_wkv7_fwd(hiprwkv_stream stream, int io_dtype, int state_dtype,
                      int64_t B, int64_t T, int64_t H, int64_t N,
                      const void* w, const void* r, const void* k, const void* v,
                      const void* a, const void* b, const void* s,
                      const uint32_t* length, const uint8_t* new_starts,
-                     void* out, float* sa, void* new_s, unsigned flags);
+                     void* out, void* sa, void* new_s, unsigned flags);
 
 /* Bytes of scratch hiprwkv_wkv7_bwd needs for this shape. */
 size_t hiprwkv_wkv7_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t N);
@@ -98,7 +100,7 @@ int hiprwkv_wkv7_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype,
                      const void* w, const void* r, const void* k, const void* v,
                      const void* a, const void* b, const void* s,
                      const uint32_t* length, const uint8_t* new_starts,
-                     const void* gy, const float* sa, const void* gs_out,
+                     const void* gy, const void* sa, const void* gs_out,
                      void* gw, void* gr, void* gk, void* gv, void* ga, void* gb, void* gs,
                      void* workspace, size_t workspace_bytes, unsigned flags);
 

@@ -108,7 +108,7 @@ int hiprwkv_handshake_failures(hiprwkv_stream stream, unsigned* count) {
 
 int hiprwkv_wkv7_fwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64_t B, int64_t T, int64_t H, int64_t N,
                      const void* w, const void* r, const void* k, const void* v, const void* a, const void* b,
-                     const void* s, const uint32_t* length, const uint8_t* new_starts, void* out, float* sa,
+                     const void* s, const uint32_t* length, const uint8_t* new_starts, void* out, void* sa,
                      void* new_s, unsigned flags) {
   int rc = check_matrix_shape("wkv7_fwd", io_dtype, state_dtype, B, T, H, N);
   if (rc) return rc;
@@ -145,7 +145,7 @@ size_t hiprwkv_wkv7_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t
 
 int hiprwkv_wkv7_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64_t B, int64_t T, int64_t H, int64_t N,
                      const void* w, const void* r, const void* k, const void* v, const void* a, const void* b,
-                     const void* s, const uint32_t* length, const uint8_t* new_starts, const void* gy, const float* sa,
+                     const void* s, const uint32_t* length, const uint8_t* new_starts, const void* gy, const void* sa,
                      const void* gs_out, void* gw, void* gr, void* gk, void* gv, void* ga, void* gb, void* gs,
                      void* workspace, size_t workspace_bytes, unsigned flags) {
   int rc = check_matrix_shape("wkv7_bwd", io_dtype, state_dtype, B, T, H, N);

@@ -44,6 +44,21 @@ __device__ __forceinline__ void st8(bf16_t* p, const float (&o)[8]) {
   *reinterpret_cast<uint4*>(p) = make_uint4(w[0], w[1], w[2], w[3]);
 }
 
+// IEEE half: the forward residual sa of the bf16 paths (11 significant bits where bf16 has 8)
+__device__ __forceinline__ void ld8(const _Float16* p, float (&o)[8]) {
+  typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
+  const h8_t a = *reinterpret_cast<const h8_t*>(p);
+#pragma unroll
+  for (int i = 0; i < 8; ++i) o[i] = (float)a[i];
+}
+__device__ __forceinline__ void st8(_Float16* p, const float (&o)[8]) {
+  typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
+  h8_t a;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) a[i] = (_Float16)o[i];
+  *reinterpret_cast<h8_t*>(p) = a;
+}
+
 // 16 consecutive elements starting at element `el` of a typed array -> 16 floats
 template <typename T>
 __device__ __forceinline__ void ld16(const void* base, size_t el, float (&o)[16]) {

@@ -27,7 +27,7 @@ enum VecKind : int {
 
 struct VecIn {
   const void* p;  // (B,T,H,64)
-  int f32;        // element type: 1 = float, 0 = bf16
+  int f32;        // element type: 1 = float, 0 = bf16, 2 = IEEE half
   int kind;       // VecKind
   int per_head;   // 1: p is (H,64), the same vector for every token and sequence
 };
@@ -37,11 +37,13 @@ struct VecOut {
 };
 
 __device__ __forceinline__ void ld8_any(const VecIn& v, size_t off, float (&o)[8]) {
-  if (v.f32) ld8(reinterpret_cast<const float*>(v.p) + off, o);
+  if (v.f32 == 1) ld8(reinterpret_cast<const float*>(v.p) + off, o);
+  else if (v.f32 == 2) ld8(reinterpret_cast<const _Float16*>(v.p) + off, o);
   else ld8(reinterpret_cast<const bf16_t*>(v.p) + off, o);
 }
 __device__ __forceinline__ void st8_any(const VecOut& v, size_t off, const float (&o)[8]) {
-  if (v.f32) st8(reinterpret_cast<float*>(v.p) + off, o);
+  if (v.f32 == 1) st8(reinterpret_cast<float*>(v.p) + off, o);
+  else if (v.f32 == 2) st8(reinterpret_cast<_Float16*>(v.p) + off, o);
   else st8(reinterpret_cast<bf16_t*>(v.p) + off, o);
 }
 __device__ __forceinline__ float vec_transform(int kind, float x) {

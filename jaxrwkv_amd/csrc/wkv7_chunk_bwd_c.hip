@@ -65,7 +65,8 @@ struct __attribute__((aligned(16))) SnapSlot {
 // Lane (t = lane%16, g = lane/16) owns token t and, of every 64-vector, the elements {8g..8g+7} u {32+8g..32+8g+7}.
 struct Raw {
   uint4 w[2], r[2], a[2], v[2], dy[2];
-  float4 sa[2][2], dsa[2][2];
+  uint4 sa[2];             // the forward residual, fp16
+  float4 dsa[2][2];
 };
 
 __device__ __forceinline__ void load_raw(Raw& x, const Wkv7Args& A, int64_t b, int64_t h, int64_t c0, int lane) {
@@ -83,12 +84,12 @@ __device__ __forceinline__ void load_raw(Raw& x, const Wkv7Args& A, int64_t b, i
       o[1][1] = *reinterpret_cast<const float4*>(p + el + 36);
     };
     ld(A.w, x.w); ld(A.r, x.r); ld(A.a, x.a); ld(A.v, x.v); ld(A.gy, x.dy);
-    ld32(A.sa_in, x.sa); ld32(A.dsa, x.dsa);
+    ld(A.sa_in, x.sa); ld32(A.dsa, x.dsa);
   } else {
     const uint4 z = make_uint4(0, 0, 0, 0);
     const float4 zf = make_float4(0.f, 0.f, 0.f, 0.f);
     x.w[0] = x.w[1] = x.r[0] = x.r[1] = x.a[0] = x.a[1] = x.v[0] = x.v[1] = x.dy[0] = x.dy[1] = z;
-    x.sa[0][0] = x.sa[0][1] = x.sa[1][0] = x.sa[1][1] = zf;
+    x.sa[0] = x.sa[1] = z;
     x.dsa[0][0] = x.dsa[0][1] = x.dsa[1][0] = x.dsa[1][1] = zf;
   }
 }
@@ -104,6 +105,17 @@ __device__ __forceinline__ void split8(const float4 lo4, const float4 hi4, u32x4
   split2(lo4.z, lo4.w, a, b); h[1] = a; l[1] = b;
   split2(hi4.x, hi4.y, a, b); h[2] = a; l[2] = b;
   split2(hi4.z, hi4.w, a, b); h[3] = a; l[3] = b;
+}
+
+// the same for eight fp16 values (11 significant bits: the pair is exact)
+__device__ __forceinline__ void split8h(const uint4 raw, u32x4_t& h, u32x4_t& l) {
+  typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
+  const h8_t x = __builtin_bit_cast(h8_t, raw);
+  uint32_t a, b;
+  split2((float)x[0], (float)x[1], a, b); h[0] = a; l[0] = b;
+  split2((float)x[2], (float)x[3], a, b); h[1] = a; l[1] = b;
+  split2((float)x[4], (float)x[5], a, b); h[2] = a; l[2] = b;
+  split2((float)x[6], (float)x[7], a, b); h[3] = a; l[3] = b;
 }
 
 __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const ChunkFlags& F, Slot* __restrict__ slot,
@@ -226,7 +238,7 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
       if (drop_dy) dr = make_uint4(0, 0, 0, 0);
       const u32x4_t dyop = {dr.x, dr.y, dr.z, dr.w};
       u32x4_t sa_h, sa_l, ds_h, ds_l;
-      split8(x.sa[hf][0], x.sa[hf][1], sa_h, sa_l);
+      split8h(x.sa[hf], sa_h, sa_l);
       split8(x.dsa[hf][0], x.dsa[hf][1], ds_h, ds_l);
       put(slot->V[t], vop, row_keep);
       put(slot->SA[0][t], sa_h, row_keep);

@@ -399,7 +399,7 @@ __device__ __forceinline__ u32x4_t load_upd(const uint16_t (*bk)[CK][RS], int ti
 struct OutCursor {
   char* y;             // A.out at (b, c0, h, 0)
   char* sa;            // A.sa (or null) at the same place
-  size_t tok_bytes;    // bytes between consecutive tokens in y (twice that in sa)
+  size_t tok_bytes;    // bytes between consecutive tokens in y and in sa
   uint32_t voff;       // lane part of the address, in elements: (4g * H) * 64 + value
 };
 
@@ -506,10 +506,12 @@ __device__ __forceinline__ bool consume(Consumer& C, Ops& o, const Slot* __restr
     *reinterpret_cast<uint16_t*>(yl + oc.tok_bytes) = (uint16_t)(y01 >> 16);
     *reinterpret_cast<uint16_t*>(yl + 2 * oc.tok_bytes) = (uint16_t)(y23 & 0xffffu);
     *reinterpret_cast<uint16_t*>(yl + 3 * oc.tok_bytes) = (uint16_t)(y23 >> 16);
-    if (oc.sa != nullptr) {
-      char* const sl = oc.sa + (size_t)oc.voff * 4;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) *reinterpret_cast<float*>(sl + 2 * i * oc.tok_bytes) = SA[i];
+    if (oc.sa != nullptr) {      // the residual for the backward pass, in fp16 like the operand it was used as
+      char* const sl = oc.sa + (size_t)oc.voff * 2;
+      *reinterpret_cast<uint16_t*>(sl) = (uint16_t)(sp[0] & 0xffffu);
+      *reinterpret_cast<uint16_t*>(sl + oc.tok_bytes) = (uint16_t)(sp[0] >> 16);
+      *reinterpret_cast<uint16_t*>(sl + 2 * oc.tok_bytes) = (uint16_t)(sp[1] & 0xffffu);
+      *reinterpret_cast<uint16_t*>(sl + 3 * oc.tok_bytes) = (uint16_t)(sp[1] >> 16);
     }
   } else {
     rare_path();
@@ -518,12 +520,16 @@ __device__ __forceinline__ bool consume(Consumer& C, Ops& o, const Slot* __restr
       if (4 * g + i < nvalid) {
         const uint32_t yv = (i & 2) ? y23 : y01;
         *reinterpret_cast<uint16_t*>(yl + i * oc.tok_bytes) = (uint16_t)((i & 1) ? (yv >> 16) : (yv & 0xffffu));
-        if (oc.sa != nullptr) *reinterpret_cast<float*>(oc.sa + (size_t)oc.voff * 4 + 2 * i * oc.tok_bytes) = SA[i];
+        if (oc.sa != nullptr) {
+          const uint32_t sv2 = sp[i >> 1];
+          *reinterpret_cast<uint16_t*>(oc.sa + (size_t)oc.voff * 2 + i * oc.tok_bytes) =
+              (uint16_t)((i & 1) ? (sv2 >> 16) : (sv2 & 0xffffu));
+        }
       }
     }
   }
   oc.y += CK * oc.tok_bytes;
-  if (oc.sa != nullptr) oc.sa += 2 * CK * oc.tok_bytes;
+  if (oc.sa != nullptr) oc.sa += CK * oc.tok_bytes;
   return ok;
 }
 
@@ -575,7 +581,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_fwd_kernel(Wkv7Args
     oc.tok_bytes = (size_t)A.H * 64 * 2;
     const size_t el0 = (((size_t)b * A.T) * A.H + h) * 64;
     oc.y = reinterpret_cast<char*>(A.out) + el0 * 2;
-    oc.sa = A.sa ? reinterpret_cast<char*>(A.sa) + el0 * 4 : nullptr;
+    oc.sa = A.sa ? reinterpret_cast<char*>(A.sa) + el0 * 2 : nullptr;
     oc.voff = (uint32_t)((4 * (lane >> 4)) * (int)A.H * 64 + 16 * cq + (lane & 15));
     const int csnap = L >= 1 ? (int)((L - 1) / CK) : -1;
     Ops ops;
@@ -617,7 +623,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_fwd_kernel(Wkv7Args
   __syncthreads();
   if (head_broken(sy, A.status)) {
     poison_token_rows(A.out, 2, b, h, A.T, A.H);
-    poison_token_rows(A.sa, 4, b, h, A.T, A.H);
+    poison_token_rows(A.sa, 2, b, h, A.T, A.H);
     poison_state(A.new_s, A.st_f32, b, h, A.H);
   }
 }

@@ -546,7 +546,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_fwd_f32_kernel(Wkv7
     oc.tok = (size_t)A.H * 64;
     const size_t el0 = (((size_t)b * A.T) * A.H + h) * 64;
     oc.y = reinterpret_cast<float*>(A.out) + el0;
-    oc.sa = A.sa ? A.sa + el0 : nullptr;
+    oc.sa = A.sa ? reinterpret_cast<float*>(A.sa) + el0 : nullptr;
     oc.voff = (uint32_t)((4 * (lane >> 4)) * (int)A.H * 64 + 16 * cq + (lane & 15));
     const int csnap = L >= 1 ? (int)((L - 1) / CK) : -1;
     Ops ops;

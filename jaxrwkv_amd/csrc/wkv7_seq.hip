@@ -116,7 +116,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void wkv7_seq_fwd_kernel(Wkv7Args A) {
   const int io = A.io_f32;
   VecIn in[6] = {{A.w, io, VK_EXPNEGEXP}, {A.r, io, VK_ID}, {A.k, io, VK_ID},
                  {A.v, io, VK_ID},        {A.a, io, VK_ID}, {A.b, io, VK_ID}};
-  VecOut out[2] = {{A.out, io}, {A.sa, 1}};
+  VecOut out[2] = {{A.out, io}, {A.sa, io ? 1 : 2}};
   seq_run<6, 2, FWD_CH, false>(st, in, out, st.id.b, st.id.h, A.T, A.H, A.ns ? A.ns + st.id.b * A.T : nullptr, smem);
 }
 
@@ -248,7 +248,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void wkv7_seq_bwd_b_kernel(Wkv7Args A)
   for (int c = 0; c < 16; ++c) st.S[c] = ld_state(A.s, A.st_f32, base + (size_t)(st.id.q * 16 + c) * N64 + st.id.line);
   const int io = A.io_f32;
   VecIn in[9] = {{A.w, io, VK_EXPNEGEXP}, {A.r, io, VK_ID}, {A.k, io, VK_ID}, {A.v, io, VK_ID}, {A.a, io, VK_ID},
-                 {A.b, io, VK_ID},        {A.gy, io, VK_ID}, {A.sa_in, 1, VK_ID}, {A.dsa, 1, VK_ID}};
+                 {A.b, io, VK_ID},        {A.gy, io, VK_ID}, {A.sa_in, io ? 1 : 2, VK_ID}, {A.dsa, 1, VK_ID}};
   VecOut out[4] = {{A.gr, io}, {A.ga, io}, {A.e2, 1}, {A.e3, 1}};
   seq_run<9, 4, BWB_CH, false>(st, in, out, st.id.b, st.id.h, A.T, A.H, A.ns ? A.ns + st.id.b * A.T : nullptr, smem);
 }
@@ -315,7 +315,7 @@ __global__ __launch_bounds__(SEQ_THREADS) void wkv7_seq_bwd_c_kernel(Wkv7Args A)
   const int io = A.io_f32;
   VecIn in[12] = {{A.w, io, VK_EXPNEGEXP}, {A.w, io, VK_NEGEXP}, {A.r, io, VK_ID},    {A.k, io, VK_ID},
                   {A.v, io, VK_ID},        {A.a, io, VK_ID},     {A.b, io, VK_ID},    {A.gy, io, VK_ID},
-                  {A.sa_in, 1, VK_ID},     {A.dsa, 1, VK_ID},    {A.e2, 1, VK_ID},    {A.e3, 1, VK_ID}};
+                  {A.sa_in, io ? 1 : 2, VK_ID},     {A.dsa, 1, VK_ID},    {A.e2, 1, VK_ID},    {A.e3, 1, VK_ID}};
   VecOut out[3] = {{A.gk, io}, {A.gb, io}, {A.gw, io}};
   seq_run<12, 3, BWC_CH, true>(st, in, out, st.id.b, st.id.h, A.T, A.H, A.ns ? A.ns + st.id.b * A.T : nullptr, smem);
 }

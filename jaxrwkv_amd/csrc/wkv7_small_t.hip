@@ -69,7 +69,10 @@ __global__ __launch_bounds__(256) void wkv7_small_t_kernel(Wkv7Args A) {
     if (compat && t + 1 < A.T && ns != nullptr && ns[t + 1]) y = 0.f;   // rwkv7.py:331-333, 344
     if (q == 0) {
       st_f(reinterpret_cast<IO*>(A.out) + tel + i, y);
-      if (A.sa != nullptr) A.sa[tel + i] = sa;
+      if (A.sa != nullptr) {      // fp32 beside fp32 I/O, IEEE half beside bf16 I/O
+        if (sizeof(IO) == 4) reinterpret_cast<float*>(A.sa)[tel + i] = sa;
+        else reinterpret_cast<_Float16*>(A.sa)[tel + i] = (_Float16)sa;
+      }
     }
     if (t == L - 1) st16<ST>(A.new_s, sel, S, q2drop);
   }

@@ -13,13 +13,13 @@ struct Wkv7Args {
   const uint32_t* length;
   const uint8_t* ns;
   void* out;
-  float* sa;      // forward residual (may be null)
+  void* sa;       // forward residual (may be null): fp32 beside fp32 I/O, IEEE half beside bf16 I/O
   void* new_s;
   int io_f32, st_f32;
   unsigned flags;
   // backward only
   const void* gy;
-  const float* sa_in;
+  const void* sa_in;     // the forward residual, in the forward's type
   const void* gs_out;
   void *gw, *gr, *gk, *gv, *ga, *gb, *gs;
   float *dsa, *e2, *e3;  // workspace, (B,T,H,64) fp32 each (the chunked sweeps keep e3_t + e2_{t+1} in e2, e3 unused)

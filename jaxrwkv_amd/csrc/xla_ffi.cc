@@ -40,20 +40,20 @@ ffi::Error status(int rc) {
 ffi::Error Wkv7Fwd(hipStream_t stream, ffi::AnyBuffer w, ffi::AnyBuffer r, ffi::AnyBuffer k, ffi::AnyBuffer v,
                    ffi::AnyBuffer a, ffi::AnyBuffer b, ffi::AnyBuffer s, ffi::Buffer<ffi::U32> length,
                    ffi::Buffer<ffi::PRED> new_starts, ffi::Result<ffi::AnyBuffer> out,
-                   ffi::Result<ffi::Buffer<ffi::F32>> sa, ffi::Result<ffi::AnyBuffer> new_s, int64_t flags) {
+                   ffi::Result<ffi::AnyBuffer> sa, ffi::Result<ffi::AnyBuffer> new_s, int64_t flags) {
   int64_t B, T, H, N;
   if (!split_thn(r.dimensions(), B, T, H, N)) return ffi::Error(ffi::ErrorCode::kInvalidArgument, "wkv7: rank < 3");
   return status(hiprwkv_wkv7_fwd(stream, dtype_of(r.element_type()), dtype_of(s.element_type()), B, T, H, N,
                                  w.untyped_data(), r.untyped_data(), k.untyped_data(), v.untyped_data(),
                                  a.untyped_data(), b.untyped_data(), s.untyped_data(), length.typed_data(),
                                  reinterpret_cast<const uint8_t*>(new_starts.typed_data()), out->untyped_data(),
-                                 sa->typed_data(), new_s->untyped_data(), static_cast<unsigned>(flags)));
+                                 sa->untyped_data(), new_s->untyped_data(), static_cast<unsigned>(flags)));
 }
 
 // operands w,r,k,v,a,b,s,length,new_starts,gy,sa,gs_out -> gw,gr,gk,gv,ga,gb,gs,workspace   (rwkv7.py:406-408)
 ffi::Error Wkv7Bwd(hipStream_t stream, ffi::AnyBuffer w, ffi::AnyBuffer r, ffi::AnyBuffer k, ffi::AnyBuffer v,
                    ffi::AnyBuffer a, ffi::AnyBuffer b, ffi::AnyBuffer s, ffi::Buffer<ffi::U32> length,
-                   ffi::Buffer<ffi::PRED> new_starts, ffi::AnyBuffer gy, ffi::Buffer<ffi::F32> sa, ffi::AnyBuffer gs_out,
+                   ffi::Buffer<ffi::PRED> new_starts, ffi::AnyBuffer gy, ffi::AnyBuffer sa, ffi::AnyBuffer gs_out,
                    ffi::Result<ffi::AnyBuffer> gw, ffi::Result<ffi::AnyBuffer> gr, ffi::Result<ffi::AnyBuffer> gk,
                    ffi::Result<ffi::AnyBuffer> gv, ffi::Result<ffi::AnyBuffer> ga, ffi::Result<ffi::AnyBuffer> gb,
                    ffi::Result<ffi::AnyBuffer> gs, ffi::Result<ffi::Buffer<ffi::U8>> workspace, int64_t flags) {
@@ -63,7 +63,7 @@ ffi::Error Wkv7Bwd(hipStream_t stream, ffi::AnyBuffer w, ffi::AnyBuffer r, ffi::
                                  w.untyped_data(), r.untyped_data(), k.untyped_data(), v.untyped_data(),
                                  a.untyped_data(), b.untyped_data(), s.untyped_data(), length.typed_data(),
                                  reinterpret_cast<const uint8_t*>(new_starts.typed_data()), gy.untyped_data(),
-                                 sa.typed_data(), gs_out.untyped_data(), gw->untyped_data(), gr->untyped_data(),
+                                 sa.untyped_data(), gs_out.untyped_data(), gw->untyped_data(), gr->untyped_data(),
                                  gk->untyped_data(), gv->untyped_data(), ga->untyped_data(), gb->untyped_data(),
                                  gs->untyped_data(), workspace->typed_data(), workspace->element_count(),
                                  static_cast<unsigned>(flags)));

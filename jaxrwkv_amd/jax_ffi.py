@@ -74,7 +74,7 @@ def wkv7_hip(r, w, k, v, a, b, s, length, new_starts):
 def _wkv7_fwd(r, w, k, v, a, b, s, length, new_starts):
     register()
     length = jnp.uint32(length)
-    out, sa, new_s = _call("hip-wkv7-fwd", (_sds(r), _sds(r, jnp.float32), _sds(s)),
+    out, sa, new_s = _call("hip-wkv7-fwd", (_sds(r), _sds(r, jnp.float32 if r.dtype == jnp.float32 else jnp.float16), _sds(s)),
                            w, r, k, v, a, b, s, length, new_starts)
     return (new_s, out), (r, w, k, v, a, b, s, length, new_starts, sa)
 

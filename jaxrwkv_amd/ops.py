@@ -11,6 +11,7 @@ import torch
 from . import _lib
 
 _DT = {torch.float32: _lib.F32, torch.bfloat16: _lib.BF16}
+_SA_DT = {torch.float32: torch.float32, torch.bfloat16: torch.float16}   # type of the WKV7 forward residual sa
 
 
 def _stream():
@@ -63,7 +64,8 @@ def handshake_failures():
 # ----------------------------------------------------------------------------- WKV7
 def wkv7_fwd(r, w, k, v, a, b, s, length=None, new_starts=None, compat=True, want_sa=False, force_seq=False,
              small_t=True, debug_flags=0):
-    """r,w,k,v,a,b (B,T,H,N) fp32|bf16; s (B,H,N,N) fp32|bf16.  Returns (new_s, y, sa|None).
+    """r,w,k,v,a,b (B,T,H,N) fp32|bf16; s (B,H,N,N) fp32|bf16.  Returns (new_s, y, sa|None); ``sa`` is fp32 for fp32
+    inputs and fp16 for bf16 inputs.
 
     T <= 8 runs on the small-T (decode) kernel unless ``small_t=False``; otherwise on a chunked matrix-core kernel
     (fp16 operands for bf16 I/O, fp32 operands for fp32 I/O); ``force_seq`` selects the sequential fp32 kernel."""
@@ -76,7 +78,8 @@ def wkv7_fwd(r, w, k, v, a, b, s, length=None, new_starts=None, compat=True, wan
     length, new_starts = _length_ns(length, new_starts, B, T, r.device)
     y = torch.empty_like(r)
     new_s = torch.empty_like(s)
-    sa = torch.empty((B, T, H, N), dtype=torch.float32, device=r.device) if want_sa else None
+    # the residual for the backward pass: fp32 beside fp32 I/O, fp16 beside bf16 I/O
+    sa = torch.empty((B, T, H, N), dtype=_SA_DT[io], device=r.device) if want_sa else None
     rc = lib.hiprwkv_wkv7_fwd(_stream(), _DT[io], _DT[s.dtype], B, T, H, N, _p(w), _p(r), _p(k), _p(v), _p(a), _p(b),
                               _p(s), _p(length), _p(new_starts), _p(y), _p(sa), _p(new_s),
                               _flags(compat, force_seq, small_t, debug_flags))
@@ -93,7 +96,7 @@ def wkv7_bwd(r, w, k, v, a, b, s, length, new_starts, gy, sa, gs_out=None, compa
     io = r.dtype
     r, w, k, v, a, b, gy = (_dev(x, io) for x in (r, w, k, v, a, b, gy))
     s = _dev(s)
-    sa = _dev(sa, torch.float32)
+    sa = _dev(sa, _SA_DT[io])
     gs_out = None if gs_out is None else _dev(gs_out, s.dtype)
     B, T, H, N = r.shape
     length, new_starts = _length_ns(length, new_starts, B, T, r.device)

@@ -108,3 +108,19 @@ def test_strong_decay_is_finite():
     x["w"][:] = 4.0
     new_s, y, sa = run(x, False)
     assert np.all(np.isfinite(y)) and np.all(np.isfinite(new_s))
+
+
+def test_values_beyond_the_fp16_range_are_loud_not_wrong():
+    """The bf16 forward feeds fp16 operands to the matrix cores: v (and with it the state) beyond 65504 cannot be
+    represented.  The conversion overflows to infinity, so y comes back non-finite instead of plausible-but-wrong;
+    the sequential kernel (HIPRWKV_FORCE_SEQ) has no such limit and still matches the oracle."""
+    from jaxrwkv_amd import ops
+    x = wkv7_inputs(1, 64, 1, 64, seed=77, bf16=True, resets=False, lengths=False)
+    x["v"] = bf16_round(x["v"] * 1.0e5).astype(np.float64)
+    t = {n: dev(x[n], torch.bfloat16) for n in "rwkvab"}
+    _, y, _ = ops.wkv7_fwd(t["r"], t["w"], t["k"], t["v"], t["a"], t["b"], dev(x["s"]), small_t=False)
+    assert not bool(torch.isfinite(y.float()).all())
+    new_s, y, _ = ops.wkv7_fwd(t["r"], t["w"], t["k"], t["v"], t["a"], t["b"], dev(x["s"]), small_t=False, force_seq=True)
+    ref_s, ref_y = o7.wkv7_base(*[x[n] for n in "rwkvab"], x["s"], x["length"], x["new_starts"], compat=True)
+    assert_close("y", host(y), ref_y, rtol=2.0 ** -7, atol=1e-4, scale_atol=True)
+    assert_close("new_s", host(new_s), ref_s, rtol=1e-4, atol=1e-4, scale_atol=True)
