@@ -1,48 +1,38 @@
-// WKV7 chunked MFMA kernels for bf16 I/O on gfx950: the forward pass and the first (reverse) sweep of the backward.
+// WKV7 backward for bf16 I/O on gfx950, first (reverse) sweep: gv, the workspace dsa and gs, 16 tokens at a time on
+// the matrix cores.
 //
-// Forward.  Recurrence per head (reference: /root/reference/src/jaxrwkv/rwkv7.py:200-220), S[i][j] = value row i,
-// key col j:
-//     sa_t = S_{t-1} a_t ;  S_t = S_{t-1} diag(d_t) + sa_t b_t^T + v_t k_t^T ;  y_t = S_t r_t ;  d_t = exp(-exp(w_t))
-// A chunk of C = 16 tokens entering with state S0 is evaluated in closed form.  With l_t = log d_t,
-// Lc_t = sum_{s<=t} l_s, E_t = exp(Lc_t), Ee_t = exp(Lc_{t-1}) and the scaled operands
+// Forward recurrence per head (reference: /root/reference/src/jaxrwkv/rwkv7.py:200-220), S[i][j] = value row i, key
+// col j:  sa_t = S_{t-1} a_t ;  S_t = S_{t-1} diag(d_t) + sa_t b_t^T + v_t k_t^T ;  y_t = S_t r_t ;  d_t = exp(-exp(w_t)).
+// With G = dL/dS carried from the last token down (G~_t the cotangent of S_t):
+//     G~_t = dy_t r_t^T + G~_{t+1} diag(d_{t+1}) + dsa_{t+1} a_{t+1}^T ;  dsa_t = G~_t b_t ;  dv_t = G~_t k_t
+// With l_t = log d_t, Lc_t = sum_{s<=t} l_s, E_t = exp(Lc_t), Ee_t = exp(Lc_{t-1}) and the scaled operands
 //     at_t = a_t.Ee_t   qt_t = r_t.E_t   kh_s = k_s/E_s   bh_s = b_s/E_s          (. and / elementwise over keys)
 //     Mba[s][t] = bh_s.at_t (s<t)   Mka[s][t] = kh_s.at_t (s<t)   Mbr[s][t] = bh_s.qt_t (s<=t)   Mkr likewise
-//     W  = S0 At^T + V^T Mka          (value x token)
-//     SA = W (I - Mba)^{-1}            sa_t for the 16 tokens; the inverse of a unit triangular 16x16
-//     Y  = S0 Qt^T + SA Mbr + V^T Mkr
-//     S_C = (S0 + SA Bh + V^T Kh) diag(E_C)
-// (I - M)^{-1} = (I + M^8)(I + M^4)(I + M^2)(I + M) because M^16 = 0.  Every product runs on
-// v_mfma_f32_16x16x32_bf16.  fp32 operands are fed as a truncated-bf16 "hi" plus a bf16 "lo" part and the three
-// significant partial products are accumulated (hi.hi + hi.lo + lo.hi), which keeps ~16 mantissa bits; the
-// doubling chain of the inverse alone runs in single bf16 (its result is split again).  The K = 32 slots of one
-// MFMA hold two 16-token products side by side.  The state stays in fp32 accumulator registers for the whole
-// sequence, transposed (key x value tiles), so that accumulator registers are reused directly as B operands.
-//
-// Reverse sweep (REV).  With G = dL/dS carried from the last token down (G~_t the cotangent of S_t):
-//     G~_t = dy_t r_t^T + G~_{t+1} diag(d_{t+1}) + dsa_{t+1} a_{t+1}^T ;  dsa_t = G~_t b_t ;  dv_t = G~_t k_t
-// Inside a chunk leaving with G_C (cotangent of the chunk-end state from later chunks), Gh = G_C diag(E_C):
+// a chunk leaving with G_C (cotangent of the chunk-end state from later chunks), Gh = G_C diag(E_C), gives
 //     G~_t diag(E_t) = Gh + sum_{s>=t} dy_s qt_s^T + sum_{s>t} dsa_s at_s^T
 //     U   = Gh Bh^T + DY^T Mbr^T         DSA = U (I - Mba^T)^{-1}         DV = Gh Kh^T + DSA Mka^T + DY^T Mkr^T
 //     G_prev = Gh + DSA At + DY^T Qt      (cotangent of the state entering the chunk)
-// which is the forward computation with the operands exchanged (Bh <-> At, Kh <-> Qt, V <-> DY, every Gram tile
-// transposed) and the decay applied before instead of after the update; the same code runs both.
+// which is the forward chunk computation with the operands exchanged (Bh <-> At, Kh <-> Qt, V <-> DY, every Gram
+// tile transposed) and the decay applied before instead of after the update.
+// (I - M)^{-1} = (I + M^8)(I + M^4)(I + M^2)(I + M) because M^16 = 0.  Every product runs on
+// v_mfma_f32_16x16x32_bf16.  fp32 operands are fed as a truncated-bf16 "hi" plus a bf16 "lo" part and the three
+// significant partial products are accumulated (hi.hi + hi.lo + lo.hi), which keeps ~16 mantissa bits; the
+// doubling chain of the inverse alone runs in single bf16 (its result is split again).  Cotangents have no bounded
+// range, so the fp16 operands of the forward kernel (wkv7_fwd.hip) are not used here.  The K = 32 slots of one MFMA
+// hold two 16-token products side by side.  G stays in fp32 accumulator registers for the whole sequence,
+// transposed (key x value tiles), so that accumulator registers are reused directly as B operands.
 //
 // Work split: one workgroup of 8 waves per (sequence, head).  Waves 0-3 are consumers: wave q owns value rows
-// 16q..16q+15 of the state and runs the state-dependent part of every chunk.  Waves 4-7 are producers: producer p
-// prepares chunks p, p+4, p+8, ... (everything that does not depend on the state: decay scan, scaled operands,
+// 16q..16q+15 of G and runs the G-dependent part of every chunk.  Waves 4-7 are producers: producer p prepares
+// chunks p, p+4, p+8, ... counted from the end (everything that does not depend on G: decay scan, scaled operands,
 // Gram tiles, triangular inverse, operand transposes) into a ring of LDS slots, four chunk periods ahead of the
-// consumers.  Synchronisation is a pair of LDS sequence numbers per slot: `ready` (set by the producer when a
-// chunk is complete) and `consumed` (one per consumer wave, set when it has read the slot for the last time).
-// Waiting is a bounded poll, so that a broken hand-shake ends the kernel (with wrong results) instead of
-// hanging the GPU.
+// consumers.  Synchronisation is a pair of LDS sequence numbers per slot with bounded waits (chunk_common.h).
 // new_starts inside a chunk restart the cumulative decay and mask the Gram tiles (rare, uniform branch).
-// The one chunk that holds token length-1 uses a second, masked operand set: for the state snapshot in the
-// forward pass, for the entry of the returned state's cotangent in the reverse sweep.
+// The one chunk that holds token length-1 uses a second, masked set of row operands through which the cotangent of
+// the returned state enters.
 //
 // Range: a key channel whose total log decay over a 16-token chunk is below -80 gets its steps of that chunk scaled
-// to a total of -80, so that 1/E_s stays finite in fp32: finite and well ordered, but no longer exact for that channel
-// (a decay of e^-5 per token sustained over a whole chunk; RWKV-7 keeps d >= 0.54 per token, i.e. e^-10 per chunk).
-// The sequential kernels have no such limit.
+// to a total of -80, so that 1/E_s stays finite in fp32 (cap_chunk_decay), as in the forward kernel.
 #include "chunk_common.h"
 #include "wkv_args.h"
 
@@ -59,8 +49,8 @@ constexpr int RING = 5;           // slots in flight
 // the 16 bytes that the same lane of a consumer loads: accumulator-layout registers (column lane%16, rows
 // 4*(lane/16)..+3) packed to bf16, hi pair then lo pair, which is exactly an A operand (row lane%16, k-slots
 // 4*(lane/16)..+3 of the hi part followed by the same slots of the lo part).
-// Names are the forward ones; the reverse sweep stores (Bh, Kh) rows in AQ, (at, qt)^T in BT, dy^T in VT and the
-// transposed Gram tiles (inverse, Mbr^T, Mka^T, Mkr^T) in Mt.
+// Names are those of the forward chunk computation; this sweep stores (Bh, Kh) rows in AQ, (at, qt)^T in BT, dy^T in
+// VT and the transposed Gram tiles (inverse, Mbr^T, Mka^T, Mkr^T) in Mt.
 struct __attribute__((aligned(16))) Slot {
   // At = a_t.Ee_t and Qt = r_t.E_t, [hi|lo][At|Qt][token][RS]: within a row, the 16-byte vector (j, g) at element
   // 32j + 8g holds keys 32j+4g..+3 followed by keys 32j+16+4g..+3, the key order of the consumers' state tiles.
@@ -72,18 +62,12 @@ struct __attribute__((aligned(16))) Slot {
   float gamma[64];             // E at the chunk end
   int snap;                    // -1, or the in-chunk index of token length-1
   int keep_end;                // the carried state passes through the whole chunk (no reset in the chunk)
-  int keep_snap;               // forward: the entering state survives to the snapshot token;
-                               // reverse: the cotangent entering at token length-1 reaches the chunk start
+  int keep_snap;               // the cotangent entering at token length-1 reaches the chunk start
   int pad;
 };
-// Operands masked for token length-1; only one chunk per sequence needs them.  Forward: update operands for the
-// state snapshot.  Reverse: row operands for the cotangent of the returned state.
-template <bool REV> struct SnapSlotT;
-template <> struct __attribute__((aligned(16))) SnapSlotT<false> {
-  uint4 BT[2][4][64];
-  float gamma[64];
-};
-template <> struct __attribute__((aligned(16))) SnapSlotT<true> {
+// Row operands masked for token length-1, through which the cotangent of the returned state enters; only one chunk
+// per sequence needs them.
+struct __attribute__((aligned(16))) SnapSlot {
   uint16_t AQ[2][2][CK][RS];
   float gamma[64];
 };
@@ -92,11 +76,10 @@ template <> struct __attribute__((aligned(16))) SnapSlotT<true> {
 // Lane (t = lane%16, g = lane/16) owns token t and the keys {8g..8g+7} u {32+8g..32+8g+7}: exactly the A/B
 // operand layout of the Gram MFMAs (row/column = token, k-slots = keys), and one 16-byte global load per half.
 struct Raw {
-  uint4 r[2], w[2], k[2], v[2], a[2], b[2];   // v holds dy in the reverse sweep
+  uint4 r[2], w[2], k[2], v[2], a[2], b[2];   // v holds dy
 };
 
 // Loads always touch a valid token (the last one of the sequence for lanes beyond it); mask_raw zeroes those lanes.
-template <bool REV>
 __device__ __forceinline__ void load_raw(Raw& x, const Wkv7Args& A, int64_t b, int64_t h, int64_t c0, int lane) {
   const int t = lane & 15, g = lane >> 4;
   const int64_t tok = (c0 + t < A.T) ? c0 + t : A.T - 1;
@@ -105,7 +88,7 @@ __device__ __forceinline__ void load_raw(Raw& x, const Wkv7Args& A, int64_t b, i
     o[0] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(p) + off);
     o[1] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(p) + off + 64);
   };
-  ld(A.r, x.r); ld(A.w, x.w); ld(A.k, x.k); ld(REV ? A.gy : A.v, x.v); ld(A.a, x.a); ld(A.b, x.b);
+  ld(A.r, x.r); ld(A.w, x.w); ld(A.k, x.k); ld(A.gy, x.v); ld(A.a, x.a); ld(A.b, x.b);
 }
 __device__ __forceinline__ void mask_raw(Raw& x, int nvalid, int lane) {
   if (nvalid != CK) {
@@ -126,9 +109,8 @@ struct Producer {
 // Everything of one chunk that does not depend on the carried state.  The two 32-key halves go through the
 // same pipeline one after the other (scan, scaling, hi/lo split, LDS parking, transposes, partial Gram sums),
 // which keeps the live register set small.
-template <bool REV>
 __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const ChunkFlags& F, Slot* __restrict__ slot,
-                                        SnapSlotT<REV>* __restrict__ snap) {
+                                        SnapSlot* __restrict__ snap) {
   const int lane = P.lane, t = lane & 15, g = lane >> 4;
   const bool valid = t < F.nvalid;
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -143,16 +125,10 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
     rare_path();
     lastseg = seg_of(F.ns, 15);
     const int myseg = seg_of(F.ns, t);
-    if (!REV) {
-      row0_keep = myseg == 0;                                          // the entering state reaches this token
-      row1_keep = row0_keep && !(F.compat && ((F.ns >> (t + 1)) & 1u)); // y[t] is defined as zero before a reset
-      if (resets) keep_upd = 0xffffu & ~((1u << (31 - __builtin_clz(resets))) - 1u);   // tokens from the last reset on
-      at_reset = (resets >> t) & 1u;
-    } else {
-      row0_keep = row1_keep = myseg == lastseg;                        // the cotangent from later chunks reaches this token
-      if (resets) keep_upd = (1u << __builtin_ctz(resets)) - 1u;       // tokens before the first reset
-      drop_dy = F.compat && ((F.ns >> (t + 1)) & 1u);                  // y[t] is a constant there
-    }
+    row0_keep = row1_keep = myseg == lastseg;                        // the cotangent from later chunks reaches this token
+    if (resets) keep_upd = (1u << __builtin_ctz(resets)) - 1u;       // tokens before the first reset
+    drop_dy = F.compat && ((F.ns >> (t + 1)) & 1u);                  // y[t] is a constant there
+
     const uint32_t upto = resets & ((2u << t) - 1u);
     const int pr = upto ? 31 - __builtin_clz(upto) : 0;             // last reset at or before this token
     restart = pr > 0;
@@ -173,13 +149,13 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
 
   // Gram tiles in accumulator layout [row m = A-operand token][column n = B-operand token]
   f32x4_t Gab = zero4, GabT = zero4;   // bh_m.at_n and at_m.bh_n
-  f32x4_t G1 = zero4, G2 = zero4, G3 = zero4;   // forward: Mka, Mbr, Mkr; reverse: qt_m.bh_n, at_m.kh_n, qt_m.kh_n
+  f32x4_t G1 = zero4, G2 = zero4, G3 = zero4;   // qt_m.bh_n, at_m.kh_n, qt_m.kh_n
 #pragma unroll
   for (int hf = 0; hf < 2; ++hf) {
     // ---- v^T (dy^T) of value tiles 2hf, 2hf+1: D[token][value] = sum_k V[token][k] sel[k][value]
     {
       uint4 vr = x.v[hf];
-      if (REV && slow) {
+      if (slow) {
         rare_path();
         if (drop_dy) vr = make_uint4(0, 0, 0, 0);
       }
@@ -210,7 +186,6 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
       for (int e = 0; e < 8; ++e) {
         const float base = __shfl(E[e], seg_src, 64);   // restart the cumulative decay at the last reset
         if (restart) E[e] -= base;
-        if (!REV && at_reset) fa[e] = 0.f;              // the state entering a reset token is zero: sa = 0
       }
     }
     // ---- scaled operands and their hi/lo split
@@ -248,12 +223,12 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
       *reinterpret_cast<float4*>(gp) = make_float4(E[0], E[1], E[2], E[3]);
       *reinterpret_cast<float4*>(gp + 4) = make_float4(E[4], E[5], E[6], E[7]);
     }
-    // ---- row operands for the consumers (forward At, Qt; reverse Bh, Kh), in their key order: this lane's keys
+    // ---- row operands for the consumers (Bh, Kh), in their key order: this lane's keys
     //      8g..8g+3 and 8g+4..8g+7 of the half are the (g>>1)-th 8-byte piece of the vectors 2(g&1) and 2(g&1)+1
     //      of block j = hf
     {
-      const u32x4_t &r0h = REV ? bh_h : at_h, &r0l = REV ? bh_l : at_l;
-      const u32x4_t &r1h = REV ? kh_h : qt_h, &r1l = REV ? kh_l : qt_l;
+      const u32x4_t &r0h = bh_h, &r0l = bh_l;
+      const u32x4_t &r1h = kh_h, &r1l = kh_l;
       const int e0 = 32 * hf + 16 * (g & 1) + 4 * (g >> 1);     // element offset of the first piece
       auto put = [&](uint16_t* row, const u32x4_t v, bool keep) {
         *reinterpret_cast<uint2*>(row + e0) = keep ? make_uint2(v[0], v[1]) : make_uint2(0u, 0u);
@@ -267,21 +242,19 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
         put(slot->AQ[0][0][t], r0h, row0_keep); put(slot->AQ[1][0][t], r0l, row0_keep);
         put(slot->AQ[0][1][t], r1h, row1_keep); put(slot->AQ[1][1][t], r1l, row1_keep);
       }
-      if constexpr (REV) {
-        if (F.snap >= 0) {
-          rare_path();
-          const bool sk = (keep_snap >> t) & 1u;
-          put(snap->AQ[0][0][t], r0h, sk); put(snap->AQ[1][0][t], r0l, sk);
-          put(snap->AQ[0][1][t], r1h, sk); put(snap->AQ[1][1][t], r1l, sk);
-        }
+      if (F.snap >= 0) {
+        rare_path();
+        const bool sk = (keep_snap >> t) & 1u;
+        put(snap->AQ[0][0][t], r0h, sk); put(snap->AQ[1][0][t], r0l, sk);
+        put(snap->AQ[0][1][t], r1h, sk); put(snap->AQ[1][1][t], r1l, sk);
       }
     }
-    // ---- transposed update operands of key tiles 2hf, 2hf+1 by MFMA (forward (b/E)^T, (k/E)^T; reverse at^T,
+    // ---- transposed update operands of key tiles 2hf, 2hf+1 by MFMA (at^T,
     //      qt^T): the accumulator layout of D (lane = key, registers = 4 consecutive tokens) is the A-operand
     //      layout of the state update
     {
-      const u32x4_t &t0h = REV ? at_h : bh_h, &t0l = REV ? at_l : bh_l;
-      const u32x4_t &t1h = REV ? qt_h : kh_h, &t1l = REV ? qt_l : kh_l;
+      const u32x4_t &t0h = at_h, &t0l = at_l;
+      const u32x4_t &t1h = qt_h, &t1l = qt_l;
 #pragma unroll
       for (int x2 = 0; x2 < 2; ++x2) {
         const int tile = 2 * hf + x2;
@@ -296,13 +269,6 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
           slot->BT[0][tile][lane] = join(masked_pack(d0h, keep_upd), masked_pack(d0l, keep_upd));
           slot->BT[1][tile][lane] = join(masked_pack(d1h, keep_upd), masked_pack(d1l, keep_upd));
         }
-        if constexpr (!REV) {
-          if (F.snap >= 0) {
-            rare_path();
-            snap->BT[0][tile][lane] = join(masked_pack(d0h, keep_snap), masked_pack(d0l, keep_snap));
-            snap->BT[1][tile][lane] = join(masked_pack(d1h, keep_snap), masked_pack(d1l, keep_snap));
-          }
-        }
       }
     }
     // ---- partial Gram sums over this half's keys (accumulator layout: column n = lane%16, rows 4g..4g+3)
@@ -314,31 +280,19 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
       const u32x4_t bB = part == 1 ? bh_l : bh_h, kB = part == 1 ? kh_l : kh_h;
       Gab = mfma(bA, aB, Gab);      // [m][n] = bh_m . at_n
       GabT = mfma(aA, bB, GabT);    // [m][n] = at_m . bh_n
-      if constexpr (!REV) {
-        G1 = mfma(kA, aB, G1);      // Mka[m][n] = kh_m . at_n
-        G2 = mfma(bA, qB, G2);      // Mbr[m][n] = bh_m . qt_n
-        G3 = mfma(kA, qB, G3);      // Mkr[m][n] = kh_m . qt_n
-      } else {
-        G1 = mfma(qA, bB, G1);      // Mbr^T[m][n] = qt_m . bh_n
-        G2 = mfma(aA, kB, G2);      // Mka^T[m][n] = at_m . kh_n
-        G3 = mfma(qA, kB, G3);      // Mkr^T[m][n] = qt_m . kh_n
-      }
+      G1 = mfma(qA, bB, G1);      // Mbr^T[m][n] = qt_m . bh_n
+      G2 = mfma(aA, kB, G2);      // Mka^T[m][n] = at_m . kh_n
+      G3 = mfma(qA, kB, G3);      // Mkr^T[m][n] = qt_m . kh_n
     }
   }
-  // ---- triangular masks: forward keeps earlier rows m for column n, the reverse sweep later rows
+  // ---- triangular masks: later rows m for column n
   const int n = t;
   auto mask_tiles = [&](int i, bool lt, bool le, bool gt, bool ge) {
     Gab[i] = lt ? Gab[i] : 0.f;
     GabT[i] = gt ? GabT[i] : 0.f;
-    if constexpr (!REV) {
-      G1[i] = lt ? G1[i] : 0.f;
-      G2[i] = le ? G2[i] : 0.f;
-      G3[i] = le ? G3[i] : 0.f;
-    } else {
-      G1[i] = ge ? G1[i] : 0.f;
-      G2[i] = gt ? G2[i] : 0.f;
-      G3[i] = ge ? G3[i] : 0.f;
-    }
+    G1[i] = ge ? G1[i] : 0.f;
+    G2[i] = gt ? G2[i] : 0.f;
+    G3[i] = ge ? G3[i] : 0.f;
   };
   if (!slow) {
 #pragma unroll
@@ -348,20 +302,19 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
     }
   } else {
     rare_path();
-    const bool keepy = REV || !(F.compat && ((F.ns >> (n + 1)) & 1u));   // forward: y[n] may be defined as zero
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int m = 4 * g + i;
       const bool same = seg_of(F.ns, m) == seg_of(F.ns, n);
-      mask_tiles(i, (m < n) && same, (m <= n) && same && keepy, (m > n) && same, (m >= n) && same);
+      mask_tiles(i, (m < n) && same, (m <= n) && same, (m > n) && same, (m >= n) && same);
     }
   }
-  // ---- (I - M)^{-1} = (I + M^8)(I + M^4)(I + M^2)(I + M) in single bf16; forward M = Mba, reverse M = Mba^T
+  // ---- (I - M)^{-1} = (I + M^8)(I + M^4)(I + M^2)(I + M) in single bf16, M = Mba^T
   auto single = [&](const f32x4_t d) {
     u32x4_t o = {pack_rn(d[0], d[1]), pack_rn(d[2], d[3]), 0u, 0u};
     return o;
   };
-  f32x4_t Mp = REV ? GabT : Gab, MpT = REV ? Gab : GabT;
+  f32x4_t Mp = GabT, MpT = Gab;
   f32x4_t Pm = Mp;
 #pragma unroll
   for (int i = 0; i < 4; ++i) Pm[i] += (4 * g + i == n) ? 1.f : 0.f;
@@ -428,8 +381,8 @@ __device__ __forceinline__ void load_ops(Ops& o, const Slot* __restrict__ slot, 
 
 // Uniform output cursors of a consumer, moved by one chunk per call.
 struct OutCursor {
-  char* y;             // forward A.out, reverse A.gv, at (b, c0, h, 0)
-  char* sa;            // forward A.sa (or null), reverse A.dsa, at the same place
+  char* y;             // A.gv at (b, c0, h, 0)
+  char* sa;            // A.dsa at the same place
   size_t tok_bytes;    // bytes between consecutive tokens in y (twice that in sa)
   uint32_t voff;       // lane part of the address, in elements: (4g * H) * 64 + value
 };
@@ -457,9 +410,9 @@ __device__ __forceinline__ void store_state_tile(void* p, int f32, size_t off, c
 
 // The state-dependent part of one chunk.  `next` is the slot of the chunk handled after this one (null after the
 // last one); `next_ready` waits until its producer has published it.
-template <bool REV, class WaitNext>
+template <class WaitNext>
 __device__ __forceinline__ bool consume(Consumer& C, Ops& o, const Slot* __restrict__ slot,
-                                        const Slot* __restrict__ next, const SnapSlotT<REV>* __restrict__ snapslot,
+                                        const Slot* __restrict__ next, const SnapSlot* __restrict__ snapslot,
                                         const Wkv7Args& A, int64_t b, int64_t h, int nvalid, bool is_snap, bool q2drop,
                                         OutCursor& oc, WaitNext&& next_ready) {
   const int lane = C.lane, n = lane & 15, g = lane >> 4;
@@ -474,13 +427,12 @@ __device__ __forceinline__ bool consume(Consumer& C, Ops& o, const Slot* __restr
     gm[tile] = *reinterpret_cast<const float4*>(&slot->gamma[16 * tile + 4 * g]);
   }
   const bool keep_end = __builtin_amdgcn_readfirstlane(o.keep_end) != 0;
-  if constexpr (REV) {
-    // the cotangent of the chunk-end state, decayed over the chunk
+  // the cotangent of the chunk-end state, decayed over the chunk
 #pragma unroll
-    for (int tile = 0; tile < 4; ++tile) {
-      C.S[tile][0] *= gm[tile].x; C.S[tile][1] *= gm[tile].y; C.S[tile][2] *= gm[tile].z; C.S[tile][3] *= gm[tile].w;
-    }
+  for (int tile = 0; tile < 4; ++tile) {
+    C.S[tile][0] *= gm[tile].x; C.S[tile][1] *= gm[tile].y; C.S[tile][2] *= gm[tile].z; C.S[tile][3] *= gm[tile].w;
   }
+
   // B operands from the state: MFMA j contracts over the keys of tiles 2j and 2j+1
   u32x4_t Sh[2], Sl[2];
 #pragma unroll
@@ -501,40 +453,39 @@ __device__ __forceinline__ bool consume(Consumer& C, Ops& o, const Slot* __restr
   W = mfma(o.Ka, o.vv, W);                    // W += Mka^T V^T (hi and lo parts side by side)
   Y = mfma(o.Kr, o.vv, Y);                    // Y += Mkr^T V^T
   const u32x4_t vv = o.vv;
-  if constexpr (REV) {
-    // a reset inside the chunk cuts the cotangent of later chunks off from the chunk start
-    if (!keep_end) {
-      asm volatile("" ::: "memory");
+  // a reset inside the chunk cuts the cotangent of later chunks off from the chunk start
+  if (!keep_end) {
+    asm volatile("" ::: "memory");
 #pragma unroll
-      for (int tile = 0; tile < 4; ++tile) C.S[tile] = zero4;
-    }
-    // the cotangent of the returned state enters at token length-1 (one chunk per sequence)
-    if (is_snap) {
-      const bool keep = slot->keep_snap != 0;
+    for (int tile = 0; tile < 4; ++tile) C.S[tile] = zero4;
+  }
+  // the cotangent of the returned state enters at token length-1 (one chunk per sequence)
+  if (is_snap) {
+    const bool keep = slot->keep_snap != 0;
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        u32x4_t gh, gl;
+    for (int j = 0; j < 2; ++j) {
+      u32x4_t gh, gl;
 #pragma unroll
-        for (int x2 = 0; x2 < 2; ++x2) {
-          const int tile = 2 * j + x2;
-          f32x4_t gs = load_state_tile(A.gs_out, A.st_f32, state_off(A, b, h, C.q, lane, tile));
-          const float4 sg = *reinterpret_cast<const float4*>(&snapslot->gamma[16 * tile + 4 * g]);
-          gs[0] *= sg.x; gs[1] *= sg.y; gs[2] *= sg.z; gs[3] *= sg.w;
-          if (keep) C.S[tile] += gs;
-          uint32_t hi, lo;
-          split2(gs[0], gs[1], hi, lo); gh[2 * x2] = hi; gl[2 * x2] = lo;
-          split2(gs[2], gs[3], hi, lo); gh[2 * x2 + 1] = hi; gl[2 * x2 + 1] = lo;
-        }
-        const u32x4_t a0h = *reinterpret_cast<const u32x4_t*>(&snapslot->AQ[0][0][n][32 * j + 8 * g]);
-        const u32x4_t a0l = *reinterpret_cast<const u32x4_t*>(&snapslot->AQ[1][0][n][32 * j + 8 * g]);
-        const u32x4_t a1h = *reinterpret_cast<const u32x4_t*>(&snapslot->AQ[0][1][n][32 * j + 8 * g]);
-        const u32x4_t a1l = *reinterpret_cast<const u32x4_t*>(&snapslot->AQ[1][1][n][32 * j + 8 * g]);
-        W = mfma(a0h, gh, W); Y = mfma(a1h, gh, Y);
-        W = mfma(a0h, gl, W); Y = mfma(a1h, gl, Y);
-        W = mfma(a0l, gh, W); Y = mfma(a1l, gh, Y);
+      for (int x2 = 0; x2 < 2; ++x2) {
+        const int tile = 2 * j + x2;
+        f32x4_t gs = load_state_tile(A.gs_out, A.st_f32, state_off(A, b, h, C.q, lane, tile));
+        const float4 sg = *reinterpret_cast<const float4*>(&snapslot->gamma[16 * tile + 4 * g]);
+        gs[0] *= sg.x; gs[1] *= sg.y; gs[2] *= sg.z; gs[3] *= sg.w;
+        if (keep) C.S[tile] += gs;
+        uint32_t hi, lo;
+        split2(gs[0], gs[1], hi, lo); gh[2 * x2] = hi; gl[2 * x2] = lo;
+        split2(gs[2], gs[3], hi, lo); gh[2 * x2 + 1] = hi; gl[2 * x2 + 1] = lo;
       }
+      const u32x4_t a0h = *reinterpret_cast<const u32x4_t*>(&snapslot->AQ[0][0][n][32 * j + 8 * g]);
+      const u32x4_t a0l = *reinterpret_cast<const u32x4_t*>(&snapslot->AQ[1][0][n][32 * j + 8 * g]);
+      const u32x4_t a1h = *reinterpret_cast<const u32x4_t*>(&snapslot->AQ[0][1][n][32 * j + 8 * g]);
+      const u32x4_t a1l = *reinterpret_cast<const u32x4_t*>(&snapslot->AQ[1][1][n][32 * j + 8 * g]);
+      W = mfma(a0h, gh, W); Y = mfma(a1h, gh, Y);
+      W = mfma(a0h, gl, W); Y = mfma(a1h, gl, Y);
+      W = mfma(a0l, gh, W); Y = mfma(a1l, gh, Y);
     }
   }
+
   // At, Qt, Mka, Mkr, v^T are dead now: fetch the next chunk's into the same registers
   bool ok = true;
   if (next != nullptr) {
@@ -559,41 +510,13 @@ __device__ __forceinline__ bool consume(Consumer& C, Ops& o, const Slot* __restr
   Y = mfma(o.Br, sHH, Y);
   Y = mfma(o.Br, sL0, Y);                     // Y^T += Mbr^T SA^T
   if (next != nullptr) o.Br = *reinterpret_cast<const u32x4_t*>(&next->Mt[2][lane]);
-  if constexpr (!REV) {
-    // state snapshot for `length` (one chunk per sequence)
-    if (is_snap) {
-      const bool keep = slot->keep_snap != 0;
-#pragma unroll
-      for (int tile = 0; tile < 4; ++tile) {
-        const u32x4_t sb = *reinterpret_cast<const u32x4_t*>(&snapslot->BT[0][tile][lane]);
-        const u32x4_t sk = *reinterpret_cast<const u32x4_t*>(&snapslot->BT[1][tile][lane]);
-        f32x4_t acc = keep ? C.S[tile] : zero4;
-        acc = mfma(sb, sHH, acc);
-        acc = mfma(sk, vv, acc);
-        acc = mfma(sb, sL0, acc);
-        const float4 sg = *reinterpret_cast<const float4*>(&snapslot->gamma[16 * tile + 4 * g]);
-        acc[0] *= sg.x; acc[1] *= sg.y; acc[2] *= sg.z; acc[3] *= sg.w;
-        store_state_tile(A.new_s, A.st_f32, state_off(A, b, h, C.q, lane, tile), q2drop ? zero4 : acc);
-      }
-    }
-    // a reset inside the chunk cuts the entering state off
-    if (!keep_end) {
-      asm volatile("" ::: "memory");   // keep this a (rare, uniform) branch instead of 16 selects on the hot path
-#pragma unroll
-      for (int tile = 0; tile < 4; ++tile) C.S[tile] = zero4;
-    }
-  }
-  // state update, tile by tile: rows = keys.  forward S <- (S + Bh^T SA^T + Kh^T V^T) . gamma,
-  // reverse G <- Gh + At^T DSA^T + Qt^T DY^T
+  // update, tile by tile: rows = keys.  G <- Gh + At^T DSA^T + Qt^T DY^T
 #pragma unroll
   for (int tile = 0; tile < 4; ++tile) {
     f32x4_t acc = C.S[tile];
     acc = mfma(bt[0][tile], sHH, acc);
     acc = mfma(bt[1][tile], vv, acc);
     acc = mfma(bt[0][tile], sL0, acc);
-    if constexpr (!REV) {
-      acc[0] *= gm[tile].x; acc[1] *= gm[tile].y; acc[2] *= gm[tile].z; acc[3] *= gm[tile].w;
-    }
     C.S[tile] = acc;
   }
   // outputs: register i is token 4g+i, lanes n = 16 consecutive values
@@ -619,25 +542,19 @@ __device__ __forceinline__ bool consume(Consumer& C, Ops& o, const Slot* __restr
       }
     }
   }
-  if constexpr (!REV) {
-    oc.y += CK * oc.tok_bytes;
-    if (oc.sa != nullptr) oc.sa += 2 * CK * oc.tok_bytes;
-  } else {
-    oc.y -= CK * oc.tok_bytes;
-    oc.sa -= 2 * CK * oc.tok_bytes;
-  }
+  oc.y -= CK * oc.tok_bytes;
+  oc.sa -= 2 * CK * oc.tok_bytes;
+
   return ok;
 }
 
 }  // namespace
 
-// Chunks are handled in sequence order in the forward pass and from the last one down in the reverse sweep; step j
-// handles chunk c(j) in slot j % RING.  Producer p fills the slot once every consumer has released step j - RING,
+// Chunks are handled from the last one down; step j
+// handles chunk c(j) = nch - 1 - j in slot j % RING.  Producer p fills the slot once every consumer has released step j - RING,
 // then publishes ready = j + 1; consumers take the steps in order.  Every wait is for a strictly earlier step, so
 // the hand-shake cannot cycle.
-template <bool REV>
-__global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_kernel(Wkv7Args A) {
-  using SnapSlot = SnapSlotT<REV>;
+__global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_bwd_a_kernel(Wkv7Args A) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   Slot* slots = reinterpret_cast<Slot*>(smem_raw);
   SnapSlot* snapslot = reinterpret_cast<SnapSlot*>(smem_raw + RING * sizeof(Slot));
@@ -651,7 +568,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_kernel(Wkv7Ar
   // the returned state is the reset state there (associative-scan rule), a constant
   const bool q2drop = (A.flags & 1u) && L < A.T && A.ns != nullptr && A.ns[b * A.T + L] != 0;
   // reverse sweep: does a cotangent of the returned state enter at token length-1?
-  const bool inject = REV && A.gs_out != nullptr && !q2drop;
+  const bool inject = A.gs_out != nullptr && !q2drop;
   if (threadIdx.x < sizeof(Sync) / sizeof(int)) reinterpret_cast<int*>(sy)[threadIdx.x] = 0;
   __syncthreads();
 
@@ -662,32 +579,18 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_kernel(Wkv7Ar
     C.q = wave;
     C.lane = lane;
     const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
-    if constexpr (!REV) {
 #pragma unroll
-      for (int tile = 0; tile < 4; ++tile) C.S[tile] = load_state_tile(A.s, A.st_f32, state_off(A, b, h, wave, lane, tile));
-      // length == 0: the returned state is the input state (rwkv7.py:203), or the reset state under the associative rule
-      if (L == 0) {
-#pragma unroll
-        for (int tile = 0; tile < 4; ++tile)
-          store_state_tile(A.new_s, A.st_f32, state_off(A, b, h, wave, lane, tile), q2drop ? zero4 : C.S[tile]);
-      }
-    } else {
-#pragma unroll
-      for (int tile = 0; tile < 4; ++tile) C.S[tile] = zero4;
-    }
-    const int64_t first_tok = REV ? (int64_t)(nch - 1) * CK : 0;
+    for (int tile = 0; tile < 4; ++tile) C.S[tile] = zero4;
+
+    const int64_t first_tok = (int64_t)(nch - 1) * CK;
     OutCursor oc;
     oc.tok_bytes = (size_t)A.H * 64 * 2;
     const size_t el0 = (((size_t)b * A.T + first_tok) * A.H + h) * 64;
-    if constexpr (!REV) {
-      oc.y = reinterpret_cast<char*>(A.out) + el0 * 2;
-      oc.sa = A.sa ? reinterpret_cast<char*>(A.sa) + el0 * 4 : nullptr;
-    } else {
-      oc.y = reinterpret_cast<char*>(A.gv) + el0 * 2;
-      oc.sa = reinterpret_cast<char*>(A.dsa) + el0 * 4;
-    }
+    oc.y = reinterpret_cast<char*>(A.gv) + el0 * 2;
+    oc.sa = reinterpret_cast<char*>(A.dsa) + el0 * 4;
+
     oc.voff = (uint32_t)((4 * (lane >> 4)) * (int)A.H * 64 + 16 * wave + (lane & 15));
-    const int csnap = (L >= 1 && (!REV || inject)) ? (int)((L - 1) / CK) : -1;
+    const int csnap = (L >= 1 && inject) ? (int)((L - 1) / CK) : -1;
     Ops ops;
     bool ok = true;
     if (nch > 0) {
@@ -695,25 +598,23 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_kernel(Wkv7Ar
       load_ops(ops, &slots[0], wave, lane);
     }
     for (int j = 0; j < nch && ok; ++j) {
-      const int c = REV ? nch - 1 - j : j;
+      const int c = nch - 1 - j;
       const int nvalid = (c + 1 < nch || A.T % CK == 0) ? CK : (int)(A.T % CK);
       const int si = j % RING, sn = (j + 1) % RING;
       const Slot* next = (j + 1 < nch) ? &slots[sn] : nullptr;
-      ok = consume<REV>(C, ops, &slots[si], next, snapslot, A, b, h, nvalid, c == csnap, q2drop, oc,
+      ok = consume(C, ops, &slots[si], next, snapslot, A, b, h, nvalid, c == csnap, q2drop, oc,
                         [&]() { return wait_ready(sy, sn, j + 2); });
       // every LDS read of slot si has returned: its data went into the MFMAs above
       if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
-    if constexpr (REV) {
-      // cotangent of the input state; with length == 0 the returned state is the input state itself
-      const bool pass = L == 0 && inject;
+    // cotangent of the input state; with length == 0 the returned state is the input state itself
+    const bool pass = L == 0 && inject;
 #pragma unroll
-      for (int tile = 0; tile < 4; ++tile) {
-        const size_t off = state_off(A, b, h, wave, lane, tile);
-        f32x4_t gsv = C.S[tile];
-        if (pass) gsv += load_state_tile(A.gs_out, A.st_f32, off);
-        store_state_tile(A.gs, A.st_f32, off, gsv);
-      }
+    for (int tile = 0; tile < 4; ++tile) {
+      const size_t off = state_off(A, b, h, wave, lane, tile);
+      f32x4_t gsv = C.S[tile];
+      if (pass) gsv += load_state_tile(A.gs_out, A.st_f32, off);
+      store_state_tile(A.gs, A.st_f32, off, gsv);
     }
   } else {
     const int p = wave - NCONS;
@@ -721,18 +622,18 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_kernel(Wkv7Ar
     P.lane = lane;
     make_sel(P.sel, lane);
     Raw raw;
-    if (p < nch) load_raw<REV>(raw, A, b, h, (int64_t)(REV ? nch - 1 - p : p) * CK, lane);
+    if (p < nch) load_raw(raw, A, b, h, (int64_t)(nch - 1 - p) * CK, lane);
     for (int j = p; j < nch; j += NPROD) {
-      const int c = REV ? nch - 1 - j : j;
+      const int c = nch - 1 - j;
       const int64_t c0 = (int64_t)c * CK;
       ChunkFlags F = chunk_flags(A.ns, A.flags, A.T, b, c0, L, lane);
-      if (REV && !inject) F.snap = -1;
+      if (!inject) F.snap = -1;
       const int si = j % RING;
       Slot* slot = &slots[si];
       if (j >= RING && !wait_consumed(sy, si, j - RING + 1, lane)) break;
       mask_raw(raw, F.nvalid, lane);
-      produce<REV>(P, raw, F, slot, snapslot);
-      if (j + NPROD < nch) load_raw<REV>(raw, A, b, h, (int64_t)(REV ? c - NPROD : c + NPROD) * CK, lane);
+      produce(P, raw, F, slot, snapslot);
+      if (j + NPROD < nch) load_raw(raw, A, b, h, (int64_t)(c - NPROD) * CK, lane);
       if ((A.flags & FLAG_DROP_PUBLISH) && j + 1 == nch) break;
       // the release orders this wave's LDS writes before the sequence number
       if (lane == 0) __hip_atomic_store(&sy->ready[si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -740,30 +641,20 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_kernel(Wkv7Ar
   }
   __syncthreads();
   if (head_broken(sy, A.status)) {
-    if constexpr (!REV) {
-      poison_token_rows(A.out, 2, b, h, A.T, A.H);
-      poison_token_rows(A.sa, 4, b, h, A.T, A.H);
-      poison_state(A.new_s, A.st_f32, b, h, A.H);
-    } else {
-      poison_token_rows(A.gv, 2, b, h, A.T, A.H);
-      poison_token_rows(A.dsa, 4, b, h, A.T, A.H);
-      poison_state(A.gs, A.st_f32, b, h, A.H);
-    }
+    poison_token_rows(A.gv, 2, b, h, A.T, A.H);
+    poison_token_rows(A.dsa, 4, b, h, A.T, A.H);
+    poison_state(A.gs, A.st_f32, b, h, A.H);
   }
 }
 
-template <bool REV>
-static hipError_t launch_chunk(const Wkv7Args& A, hipStream_t stream) {
-  const size_t smem = RING * sizeof(Slot) + sizeof(SnapSlotT<REV>) + sizeof(Sync);
+// Reverse sweep of the backward pass: gv, the workspace dsa (cotangent of sa per token) and gs.
+hipError_t launch_wkv7_chunk_bwd_a(const Wkv7Args& A, hipStream_t stream) {
+  const size_t smem = RING * sizeof(Slot) + sizeof(SnapSlot) + sizeof(Sync);
   static LdsAttrOnce once;
-  const hipError_t attr = allow_dynamic_lds(once, reinterpret_cast<const void*>(wkv7_chunk_kernel<REV>), smem);
+  const hipError_t attr = allow_dynamic_lds(once, reinterpret_cast<const void*>(wkv7_bwd_a_kernel), smem);
   if (attr != hipSuccess) return attr;
-  hipLaunchKernelGGL(wkv7_chunk_kernel<REV>, dim3((unsigned)(A.B * A.H)), dim3(64 * (NCONS + NPROD)), smem, stream, A);
+  hipLaunchKernelGGL(wkv7_bwd_a_kernel, dim3((unsigned)(A.B * A.H)), dim3(64 * (NCONS + NPROD)), smem, stream, A);
   return hipGetLastError();
 }
-
-
-// Reverse sweep of the backward pass: gv, the workspace dsa (cotangent of sa per token) and gs.
-hipError_t launch_wkv7_chunk_bwd_a(const Wkv7Args& A, hipStream_t stream) { return launch_chunk<true>(A, stream); }
 
 }  // namespace hiprwkv
