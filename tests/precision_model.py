@@ -1,4 +1,5 @@
-"""NumPy model of the chunked WKV7 forward kernel with a selectable operand precision for every matrix product.
+"""NumPy models of the chunked WKV7 and WKV6 forward kernels with a selectable operand precision for every matrix
+product (WKV7 first; the WKV6 model is at the end of the file).
 
 The chunked kernel (jaxrwkv_amd/csrc/wkv7_fwd.hip) evaluates 16 tokens at a time from the entering state S0
 (recurrence: /root/reference/src/jaxrwkv/rwkv7.py:200-220).  With l_t = log d_t, Lc_t = sum_{s<=t} l_s:
@@ -168,6 +169,73 @@ ABLATION = [
 ]
 
 
+# ------------------------------------------------------------------------------------------------------ WKV6
+# The chunked WKV6 forward (jaxrwkv_amd/csrc/wkv6_fwd.hip; recurrence /root/reference/src/jaxrwkv/rwkv6.py:175-191,
+# S[key][value]):  Y = Qt S0 + M^T V,  S_C = diag(E_C) S0 + Ke^T V  with qt_t = r_t exp(Lc_{t-1}), kh_s = k_s exp(-Lc_s),
+# ke_s = k_s exp(Lc_15 - Lc_s), M[s][t] = kh_s.qt_t (s < t), M[t][t] = sum r u k.  Operand keys:
+#   s  state in Qt S0        q  qt in Qt S0        g  kh, qt in the Gram tile        m  M as the consumers read it
+#   upd  ke in the state update
+EXACT6 = dict(s="f1", q="f1", g="f1", m="f1", upd="f1")
+CHOSEN6 = dict(s="h1", q="h1", g="b2", m="h2", upd="h1")
+
+
+def chunk_forward6(r, lw, k, v, u, S0, p):
+    """One chunk for a batch of heads: token arrays (G, 16, 64), lw = log decay, u (G, 64), S0 (G, 64, 64) [key][value]."""
+    Lc = np.cumsum(lw, axis=1)
+    Le = np.concatenate([np.zeros_like(Lc[:, :1]), Lc[:, :-1]], axis=1)
+    qt, kh = r * np.exp(Le), k * np.exp(-Lc)
+    ke = k * np.exp(Lc[:, -1:] - Lc)
+    gam = np.exp(Lc[:, -1])
+    s_i, t_i = np.arange(CK)[:, None], np.arange(CK)[None, :]
+    M = mm(Q(kh, p["g"]), Q(qt, p["g"]), "gsj,gtj->gst") * (s_i < t_i)
+    M = M + np.eye(CK) * np.einsum("gtj,gj,gtj->gt", r, u, k)[:, None, :]
+    vq = Q(v, "f1")
+    Y = mm(Q(qt, p["q"]), Q(S0, p["s"]), "gtj,gji->gti") + mm(Q(M, p["m"]), vq, "gst,gsi->gti")
+    SC = S0 * gam[:, :, None] + mm(Q(ke, p["upd"]), vq, "gsj,gsi->gji")
+    return Y, SC.astype(np.float32).astype(np.float64)
+
+
+def forward6(x, p):
+    """Whole sequences without resets: x from tests.inputs.wkv6_inputs (resets=False, lengths=False)."""
+    B, T, H, N = x["r"].shape
+    assert T % CK == 0
+    f = lambda n: x[n].transpose(0, 2, 1, 3).reshape(B * H, T, N)
+    r, w, k, v = (f(n) for n in "rwkv")
+    u = np.broadcast_to(x["u"][None], (B, H, N)).reshape(B * H, N)
+    S = x["s"].reshape(B * H, N, N).astype(np.float64)
+    y = np.zeros_like(r)
+    for c0 in range(0, T, CK):
+        sl = slice(c0, c0 + CK)
+        y[:, sl], S = chunk_forward6(r[:, sl], w[:, sl], k[:, sl], v[:, sl], u, S, p)
+    return S.reshape(B, H, N, N), y.reshape(B, H, T, N).transpose(0, 2, 1, 3)
+
+
+def metrics6(x, p, ref=None):
+    from oracle import wkv6 as o6
+    from .gpu_util import tvd_of_projected
+    if ref is None:
+        ref = o6.wkv6_base(x["r"], x["k"], x["v"], x["w"], x["u"], x["s"], x["length"], x["new_starts"])
+    ref_s, ref_y = ref
+    S, y = forward6(x, p)
+    rel = lambda got, want: float(np.sqrt(np.mean((got - want) ** 2) / np.mean(want ** 2)))
+    yb, rb = bf16_round(y).astype(np.float64), bf16_round(ref_y).astype(np.float64)
+    tvd = tvd_of_projected(yb, rb)
+    return dict(y=rel(y, ref_y), s=rel(S, ref_s), flips=float(np.mean(yb != rb)), tvd_max=float(tvd.max()),
+                tvd_mean=float(tvd.mean())), ref
+
+
+ABLATION6 = [
+    ("exact operands", EXACT6),
+    ("single bf16 everywhere", dict(s="b1", q="b1", g="b1", m="b1", upd="b1")),
+    ("fp16 everywhere, bf16 pairs in the Gram tile, M an fp16 pair (chosen)", CHOSEN6),
+    ("chosen, M single fp16", {**CHOSEN6, "m": "h1"}),
+    ("chosen, Gram operands single bf16", {**CHOSEN6, "g": "b1"}),
+    ("chosen, state fp16 pair", {**CHOSEN6, "s": "h2"}),
+    ("chosen, state and qt fp16 pairs", {**CHOSEN6, "s": "h2", "q": "h2"}),
+    ("chosen, update operand single bf16", {**CHOSEN6, "upd": "b1"}),
+]
+
+
 def main():
     for regime in ("bench", "slow"):
         x = make_inputs(regime)
@@ -177,6 +245,14 @@ def main():
         for name, p in ABLATION:
             m, ref = metrics(x, p, ref)
             print(f"{name:66s} {m['y']:9.2e} {m['s']:9.2e} {m['sa']:9.2e} {m['flips']:8.4f} {m['tvd_max']:9.2e} {m['tvd_mean']:9.2e}")
+    from .inputs import wkv6_inputs
+    x = wkv6_inputs(2, 1024, 4, 64, seed=0, bf16=True, resets=False, lengths=False)
+    ref = None
+    print("\nWKV6, B=2 T=1024 H=4, bf16 inputs; errors against the float64 sequential oracle")
+    print(f"{'operand formats':72s} {'y relrms':>9s} {'S relrms':>9s} {'y flips':>8s} {'TVD max':>9s} {'TVD mean':>9s}")
+    for name, p in ABLATION6:
+        m, ref = metrics6(x, p, ref)
+        print(f"{name:72s} {m['y']:9.2e} {m['s']:9.2e} {m['flips']:8.4f} {m['tvd_max']:9.2e} {m['tvd_mean']:9.2e}")
 
 
 if __name__ == "__main__":

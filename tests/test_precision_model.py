@@ -54,3 +54,44 @@ def test_pairs_everywhere_is_two_orders_better_but_not_needed(case):
     x, ref, _ = case
     m, _ = pm.metrics(x, pm.ALL_SPLIT, ref)
     assert m["y"] < 3e-5 and m["tvd_max"] < 1e-3, m
+
+
+# ---------------------------------------------------------------------------------------------------------- WKV6
+@pytest.fixture(scope="module")
+def case6():
+    from .inputs import wkv6_inputs
+    x = wkv6_inputs(1, 512, 4, 64, seed=0, bf16=True, resets=False, lengths=False)
+    m, ref = pm.metrics6(x, pm.EXACT6)
+    return x, ref, m
+
+
+def test_wkv6_exact_operands_reproduce_the_recurrence(case6):
+    _, _, m = case6
+    assert m["y"] < 1e-6 and m["s"] < 1e-6 and m["tvd_max"] < 1e-4
+
+
+def test_wkv6_chosen_formats_meet_the_bf16_bar(case6):
+    """jaxrwkv_amd/csrc/wkv6_fwd.hip: fp16 state, qt, ke, v; bf16 pairs for the Gram operands; M as an fp16 pair."""
+    x, ref, _ = case6
+    m, _ = pm.metrics6(x, pm.CHOSEN6, ref)
+    assert m["tvd_max"] < 1e-3 and m["y"] < 2e-4 and m["s"] < 3e-4, m
+
+
+def test_wkv6_the_gram_tile_pair_is_what_keeps_y_close(case6):
+    """M carries the diagonal bonus and the nearest tokens, most of y: as a single fp16 number it triples the error
+    of y and the share of y elements that differ from the exactly rounded ones."""
+    x, ref, _ = case6
+    pair, _ = pm.metrics6(x, pm.CHOSEN6, ref)
+    single, _ = pm.metrics6(x, {**pm.CHOSEN6, "m": "h1"}, ref)
+    assert single["y"] > 2.5 * pair["y"] and single["flips"] > 3 * pair["flips"], (pair, single)
+
+
+@pytest.mark.parametrize("name,override", [
+    ("single bf16 everywhere", dict(s="b1", q="b1", g="b1", m="b1", upd="b1")),
+    ("Gram operands single bf16", {**pm.CHOSEN6, "g": "b1"}),
+    ("update operand single bf16", {**pm.CHOSEN6, "upd": "b1"}),
+])
+def test_wkv6_cheaper_formats_miss_it(case6, name, override):
+    x, ref, _ = case6
+    m, _ = pm.metrics6(x, override, ref)
+    assert m["tvd_max"] > 1e-3, (name, m)
