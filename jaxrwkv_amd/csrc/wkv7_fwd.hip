@@ -11,7 +11,9 @@
 //
 // Operand formats.  at, qt, ke, be, v, the state, W, SA, P and the three M tiles are bounded by the inputs' magnitudes:
 // they go to the matrix cores as single fp16 numbers (11 significant bits; the values must stay inside the fp16
-// range, |x| < 65504).  kh and bh carry exp(-Lc) and need the fp32 exponent range: the four Gram tiles are formed from
+// range, |x| < 65504) -- but for Mkr, which multiplies v straight into y (its diagonal is the token's own k.r) and is
+// fed as an fp16 pair hi + lo: one more K = 16 instruction per consumer and chunk for a y error 3.5 times smaller
+// where the decay is fast.  kh and bh carry exp(-Lc) and need the fp32 exponent range: the four Gram tiles are formed from
 // bf16 hi + lo pairs of kh, bh, at, qt (three partial products).  The state itself stays in fp32 accumulator
 // registers for the whole sequence, stored transposed (key x value tiles).
 //
@@ -88,6 +90,7 @@ struct __attribute__((aligned(16))) Slot {
   uint16_t V[CK][RS];          // v in fp16
   u32x2_t P[64], Ka[64];       // lane-indexed fp16: column t = lane%16, rows 4g..4g+3 (g = lane/16) of P and Mka
   u32x4_t BrKr[64];            // the same of Mbr followed by Mkr
+  u32x2_t KrLo[64];            // Mkr minus its fp16 value, in fp16: Mkr multiplies v straight into y
   float gamma[64];             // exp(Lc_15)
   int snap;                    // -1, or the in-chunk index of token length-1
   int keep_end;                // the carried state passes through the whole chunk (no reset in the chunk)
@@ -348,6 +351,11 @@ __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags
   {
     const u32x2_t br = pack_h4(G2), kr = pack_h4(G3);
     slot->BrKr[lane] = u32x4_t{br[0], br[1], kr[0], kr[1]};
+    const f16x4_t krh = __builtin_bit_cast(f16x4_t, kr);
+    f32x4_t rest;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) rest[i] = G3[i] - (float)krh[i];
+    slot->KrLo[lane] = pack_h4(rest);
   }
   if (lane == 0) {
     slot->snap = F.snap;
@@ -369,6 +377,7 @@ struct Ops {
   u32x4_t aq[2][2];        // [at|qt][j]: rows in the key order of the state tiles
   u32x2_t P, Ka;
   u32x4_t BrKr;
+  u32x2_t KrLo;
   u32x2_t vv;              // v^T of this wave's value tile: tokens 4g..4g+3 of value n
   int keep_end;
 };
@@ -383,6 +392,7 @@ __device__ __forceinline__ void load_ops(Ops& o, const Slot* __restrict__ slot, 
   o.P = slot->P[lane];
   o.Ka = slot->Ka[lane];
   o.BrKr = slot->BrKr[lane];
+  o.KrLo = slot->KrLo[lane];
   o.vv = lds_tr4(&slot->V[4 * g + (n >> 2)][16 * q + 4 * (n & 3)]);
   o.keep_end = slot->keep_end;
 }
@@ -450,7 +460,8 @@ __device__ __forceinline__ bool consume(Consumer& C, Ops& o, const Slot* __restr
   for (int j = 0; j < 2; ++j)
     Sh[j] = u32x4_t{pack_h(C.S[2 * j][0], C.S[2 * j][1]), pack_h(C.S[2 * j][2], C.S[2 * j][3]),
                     pack_h(C.S[2 * j + 1][0], C.S[2 * j + 1][1]), pack_h(C.S[2 * j + 1][2], C.S[2 * j + 1][3])};
-  f32x4_t W = zero4, Y = zero4;   // [token 4g+i][value n], two interleaved accumulation chains
+  f32x4_t W = zero4;              // [token 4g+i][value n], two interleaved accumulation chains
+  f32x4_t Y = mfma_h16(o.KrLo, o.vv, zero4);    // the low part of Mkr^T V^T: no state in it, off the critical path
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     W = mfma_h(o.aq[0][j], Sh[j], W);

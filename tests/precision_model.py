@@ -63,14 +63,16 @@ def mm(a, b, sub):
 #   s      state in W = S0 At^T and Y = S0 Qt^T          aq    At and Qt in those two products
 #   gk     kh, bh in the Gram tiles                      ga    at, qt in the Gram tiles
 #   inv    every operand of the doubling chain           m     T, Mka, Mbr, Mkr as the consumers read them
+#   mkr    Mkr alone (default: m)
 #   w      W in SA = W T                                 sa    SA in Y and in the state update
 #   upd    ke, be in the state update
 EXACT = dict(s="f1", aq="f1", gk="f1", ga="f1", inv="f1", m="f1", w="f1", sa="f1", upd="f1")
 ALL_SPLIT = dict(s="b2", aq="b2", gk="b2", ga="b2", inv="b1", m="b2", w="b2", sa="b2", upd="b2")   # the first kernel
 ALL_BF16 = dict(s="b1", aq="b1", gk="b1", ga="b1", inv="b1", m="b1", w="b1", sa="b1", upd="b1")
-# the set the kernel uses: fp16 wherever the operand is bounded by the inputs' magnitudes, bf16 pairs for the Gram
-# operands kh, bh (they carry exp(-Lc) and need the fp32 exponent range)
-CHOSEN = dict(s="h1", aq="h1", gk="b2", ga="b2", inv="h1", m="h1", w="h1", sa="h1", upd="h1")
+# the set the kernel uses: fp16 wherever the operand is bounded by the inputs' magnitudes (Mkr, which multiplies v
+# straight into y, as an fp16 pair), bf16 pairs for the Gram operands kh, bh (they carry exp(-Lc) and need the fp32
+# exponent range) and at, qt
+CHOSEN = dict(s="h1", aq="h1", gk="b2", ga="b2", inv="h1", m="h1", mkr="h2", w="h1", sa="h1", upd="h1")
 
 
 def chunk_forward(r, l, k, v, a, b, S0, p):
@@ -95,7 +97,7 @@ def chunk_forward(r, l, k, v, a, b, S0, p):
         q = Q(Mp, p["inv"])
         Mp = mm(q, q, "gsu,gut->gst")
         P = P + mm(Q(Mp, p["inv"]), Q(P, p["inv"]), "gsu,gut->gst")
-    Tq, Kaq, Brq, Krq = Q(P, p["m"]), Q(Mka, p["m"]), Q(Mbr, p["m"]), Q(Mkr, p["m"])
+    Tq, Kaq, Brq, Krq = Q(P, p["m"]), Q(Mka, p["m"]), Q(Mbr, p["m"]), Q(Mkr, p.get("mkr", p["m"]))
     Sq = Q(S0, p["s"])
     vq = Q(v, "f1")                                           # v is an input: exact in bf16 and (normal range) in fp16
     W = mm(Sq, Q(at, p["aq"]), "gij,gtj->git") + mm(vq, Kaq, "gsi,gst->git")
@@ -152,15 +154,16 @@ ABLATION = [
     ("exact operands", EXACT),
     ("bf16 pairs everywhere (inverse chain single)", ALL_SPLIT),
     ("single bf16 everywhere", ALL_BF16),
-    ("single fp16 everywhere but bf16 pairs in the Gram tiles (chosen)", CHOSEN),
+    ("fp16 everywhere, bf16 pairs in the Gram tiles, Mkr an fp16 pair (chosen)", CHOSEN),
+    ("chosen, Mkr single fp16", {**CHOSEN, "mkr": "h1"}),
     ("chosen, Gram operands single bf16", {**CHOSEN, "gk": "b1", "ga": "b1"}),
     ("chosen, Gram kh/bh pairs but at/qt single bf16", {**CHOSEN, "ga": "b1"}),
     ("chosen, state single bf16", {**CHOSEN, "s": "b1", "aq": "b1"}),
     ("chosen, state fp16 pair", {**CHOSEN, "s": "h2"}),
     ("chosen, state and At/Qt fp16 pairs", {**CHOSEN, "s": "h2", "aq": "h2"}),
     ("chosen, inverse chain single bf16", {**CHOSEN, "inv": "b1"}),
-    ("chosen, tiles T/Mka/Mbr/Mkr single bf16", {**CHOSEN, "m": "b1"}),
-    ("chosen, tiles fp16 pairs", {**CHOSEN, "m": "h2"}),
+    ("chosen, tiles T/Mka/Mbr/Mkr single bf16", {**CHOSEN, "m": "b1", "mkr": "b1"}),
+    ("chosen, all four tiles fp16 pairs", {**CHOSEN, "m": "h2"}),
     ("chosen, W single bf16", {**CHOSEN, "w": "b1"}),
     ("chosen, SA single bf16", {**CHOSEN, "sa": "b1"}),
     ("chosen, W and SA fp16 pairs", {**CHOSEN, "w": "h2", "sa": "h2"}),
