@@ -29,9 +29,9 @@ B, T, H, N = 8, 4096, 32, 64
 # figures in profiles/), each with the sha1 prefix of the kernel source it was measured on: when the source has
 # changed since, `roofline.traffic` is null instead of a stale figure.
 MEASURED_TRAFFIC = {
-    "wkv7_fwd": (948.5e6, "wkv7_fwd.hip", None),
-    "wkv4_fwd": (4028.7e6, "wkv4.hip", None),
-    "wkv6_fwd": (701.6e6, "wkv6_fwd.hip", None),
+    "wkv7_fwd": (948.5e6, "wkv7_fwd.hip", "86253aea7c44"),
+    "wkv4_fwd": (4028.7e6, "wkv4.hip", "d83a0992a92e"),
+    "wkv6_fwd": (688.5e6, "wkv6_fwd.hip", "0a029503ae09"),
 }
 
 
