@@ -475,8 +475,8 @@ __device__ __forceinline__ bool consume(Consumer& C, Ops& o, const Slot* __restr
         acc[0] = old[tile][0] * sg.x; acc[1] = old[tile][1] * sg.y;
         acc[2] = old[tile][2] * sg.z; acc[3] = old[tile][3] * sg.w;
       }
+      acc = mfma_tt(sk, vv, acc);     // the order of the update below: a snapshot at the chunk end has its bits
       acc = mfma_tt(sb, SA, acc);
-      acc = mfma_tt(sk, vv, acc);
       store_state_tile(A.new_s, A.st_f32, state_off(A, b, h, C.q, lane, tile), q2drop ? zero4 : acc);
     }
   }

@@ -53,6 +53,10 @@ def _call(target, result_types, *operands):
     # copy).  The handlers in csrc/xla_ffi.cc rely on exactly that: they take the last three (WKV4: two) dimensions
     # as (T, H, N) and fold everything before them into one flat batch B, for the state, length and new_starts
     # operands too.  An operand vmapped with a non-leading out-axis would break this; jax.ffi never produces one.
+    # The per-head / per-channel parameters (WKV6 u (H,N), WKV4 w and u (C,)) then arrive with the same leading batch
+    # shape, and the C ABI reads only the first (H,N) / (C,) of them: right when they were broadcast, which is the
+    # reference's use (one parameter set per model), and silently wrong for a caller that vmaps over per-example
+    # parameters.
     return jax.ffi.ffi_call(target, result_types, vmap_method="broadcast_all")(*operands, flags=np.int64(COMPAT_ASSOC))
 
 

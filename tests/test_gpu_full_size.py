@@ -162,3 +162,53 @@ def test_wkv7_decode_shape_of_the_1p5b_config(st):
         assert_close("new_s", host(new_s), ref_s)
     else:
         assert_close("new_s", host(new_s), ref_s, rtol=2.0 ** -8, atol=1e-6)
+
+
+def test_wkv7_fp32_chunked_equals_sequential_and_split_call_at_the_headline_shape():
+    """fp32 I/O at B=8 T=4096 H=32: the chunked kernel on fp32 matrix instructions against the sequential fp32 kernel
+    at the fp32 bar (rtol 1e-4, atol 1e-5 of the tensor's rms scale), and a split call with the carried state against
+    the single call, bit for bit."""
+    from jaxrwkv_amd import ops
+    x = wkv7_full(seed=5)
+    f = {n: x[n].float() for n in "rwkvab"}
+    args = tuple(f[n] for n in "rwkvab") + (x["s"], x["length"], x["ns"])
+    a = ops.wkv7_fwd(*args, compat=True, want_sa=True)
+    b = ops.wkv7_fwd(*args, compat=True, want_sa=True, force_seq=True)
+    torch.cuda.synchronize()
+    for name, c, q in zip(("new_s", "y", "sa"), a, b):
+        assert c.dtype == torch.float32 and torch.isfinite(c).all(), name
+        scale = float(q.pow(2).mean().sqrt())
+        excess = ((c - q).abs() - 1e-4 * q.abs()).max()
+        assert float(excess) < 1e-5 * max(1.0, scale), (name, float(excess), scale)
+    h = 2048
+    sl = lambda t, lo, hi: t[:, lo:hi].contiguous()
+    full_s, full_y, _ = ops.wkv7_fwd(*(f[n] for n in "rwkvab"), x["s"], None, x["ns"], compat=False)
+    s1, y1, _ = ops.wkv7_fwd(*(sl(f[n], 0, h) for n in "rwkvab"), x["s"], None, sl(x["ns"], 0, h), compat=False)
+    s2, y2, _ = ops.wkv7_fwd(*(sl(f[n], h, 4096) for n in "rwkvab"), s1, None, sl(x["ns"], h, 4096), compat=False)
+    torch.cuda.synchronize()
+    assert torch.equal(torch.cat([y1, y2], 1), full_y) and torch.equal(s2, full_s)
+
+
+def test_wkv4_backward_with_forward_checkpoints_at_the_benchmark_shape():
+    """B=32 T=4096 C=2560 fp32: the forward that keeps the checkpoints returns the plain forward's bits, and the
+    backward that takes them returns the bits of the backward with its own checkpoint pass."""
+    from jaxrwkv_amd import ops
+    B, T, C = 32, 4096, 2560
+    g = torch.Generator("cuda").manual_seed(6)
+    k = torch.randn((B, T, C), device="cuda", generator=g)
+    v = torch.randn((B, T, C), device="cuda", generator=g)
+    gy = torch.randn((B, T, C), device="cuda", generator=g)
+    w = -torch.exp(torch.randn(C, device="cuda", generator=g))
+    u = 0.5 * torch.randn(C, device="cuda", generator=g)
+    s = torch.zeros((B, 3, C), device="cuda")
+    s[:, 2] = -1e38
+    length = torch.randint(1024, T + 1, (B,), device="cuda", generator=g, dtype=torch.int32)
+    ns = torch.rand((B, T), device="cuda", generator=g) < 1.0 / 1024
+    plain = ops.wkv4_fwd(w, u, k, v, s, length, ns)
+    new_s, y, ck = ops.wkv4_fwd(w, u, k, v, s, length, ns, want_ckpt=True)
+    assert torch.equal(new_s, plain[0]) and torch.equal(y, plain[1])
+    own = ops.wkv4_bwd(w, u, k, v, s, length, ns, gy)
+    taken = ops.wkv4_bwd(w, u, k, v, s, length, ns, gy, ckpt=ck)
+    torch.cuda.synchronize()
+    for p_, q_ in zip(own, taken):
+        assert torch.isfinite(p_.float()).all() and torch.equal(p_, q_)
