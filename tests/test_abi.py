@@ -50,6 +50,14 @@ def test_argument_validation_without_gpu():
     rc = lib.hiprwkv_wkv4_bwd(null, 0, 1, 8, (1 << 23) + 1, *([null] * 14), null, 0, 0)
     assert rc == -1 and b"2^23" in lib.hiprwkv_last_error()
     assert lib.hiprwkv_wkv4_bwd_workspace_bytes(2, 17, 64) >= 2 * 2 * 3 * 64 * 4
+    # the forward that keeps the backward's checkpoints: workspace pointer and size are checked first
+    ok = ctypes.c_void_p(0x10000)
+    rc = lib.hiprwkv_wkv4_fwd_ckpt(null, 0, 2, 17, 64, *([ok] * 5), null, null, ok, ok, null, 1 << 20, 0)
+    assert rc == -1 and b"workspace" in lib.hiprwkv_last_error()
+    rc = lib.hiprwkv_wkv4_fwd_ckpt(null, 0, 2, 17, 64, *([ok] * 5), null, null, ok, ok, ok, 16, 0)
+    assert rc == -3 and b"needed" in lib.hiprwkv_last_error()
+    rc = lib.hiprwkv_wkv4_fwd_ckpt(null, 0, 0, 17, 64, *([ok] * 5), null, null, ok, ok, ok, 1 << 20, 0)
+    assert rc == -1
     assert lib.hiprwkv_wkv7_bwd_workspace_bytes(2, 16, 2, 64) == 3 * 2 * 16 * 2 * 64 * 4
     assert lib.hiprwkv_wkv6_bwd_workspace_bytes(2, 16, 2, 64) >= 2 * 16 * 2 * 64 * 4
 
