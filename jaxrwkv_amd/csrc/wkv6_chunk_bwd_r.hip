@@ -11,9 +11,10 @@
 //     G_t v_t   = (1/E_t) . ( Gh v_t + sum_{s>t} (dy_s.v_t) rq_s )          contracts over values
 //     G_t^T k_t = Gh^T kh_t + sum_{s>t} (rq_s.kh_t) dy_s                     contracts over keys
 //     G_prev = Gh + sum_s rq_s dy_s^T
-// The two contractions run over different axes of G, so every consumer wave keeps two accumulator copies: G1 = the
-// rows of its 16 keys (all values, for G v) and G2 = the columns of its 16 values (all keys, for G^T k); both get the
-// same rank-16 update.  Products with fp32 quantities run as hi.hi + hi.lo + lo.hi on v_mfma_f32_16x16x32_bf16.
+// The two contractions run over different axes of G, so there are two kinds of consumer wave, four of each: a key wave
+// keeps the rows of its 16 keys (all values, for G v), a value wave the columns of its 16 values (all keys, for
+// G^T k); both get the same rank-16 update.  (One wave holding both copies has twice the dependent work per chunk and
+// paces the sweep; two kinds of wave halve it, and twelve waves at 160 registers still fit three to a SIMD.)  Products with fp32 quantities run as hi.hi + hi.lo + lo.hi on v_mfma_f32_16x16x32_bf16.
 // Work split, LDS ring and hand-shake as in the other chunked kernels; the producers also own the state-free terms
 // r u c_t and dy (r.(u k)), handed over as fp32 add-ons.  Range: a chunk's total log decay per channel is capped at -80.
 #include "chunk_common.h"
@@ -28,6 +29,37 @@ using namespace chunk;
 constexpr int NPROD = 4;          // producer waves; producer p owns steps p, p + NPROD, ...
 constexpr int RING = 5;           // slots in flight (a slot is 30 KB)
 constexpr int ES = 68;            // row stride (floats) of the fp32 [token][.] arrays: conflict-free column reads
+constexpr int NCONS_R = 8;        // consumer waves: 0-3 hold G1 (gk, gw, gs), 4-7 hold G2 (gv)
+
+struct __attribute__((aligned(16))) Sync8 {      // the hand-shake words of chunk_common.h for eight consumers
+  int ready[MAX_RING];
+  int consumed[NCONS_R][MAX_RING];
+  int broken;
+  int pad[3];
+};
+__device__ __forceinline__ bool wait_ready8(Sync8* sy, int slot, int want) {
+  for (int spin = 0; spin < SPIN_LIMIT; ++spin) {
+    if (__hip_atomic_load(&sy->ready[slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) == want) return true;
+    __builtin_amdgcn_s_sleep(1);
+  }
+  __hip_atomic_store(&sy->broken, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  return false;
+}
+__device__ __forceinline__ bool wait_consumed8(Sync8* sy, int slot, int want, int lane) {
+  for (int spin = 0; spin < SPIN_LIMIT; ++spin) {
+    int seen = want;
+    if (lane < NCONS_R) seen = __hip_atomic_load(&sy->consumed[lane][slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (__ballot(seen < want) == 0ull) return true;
+    __builtin_amdgcn_s_sleep(1);
+  }
+  __hip_atomic_store(&sy->broken, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  return false;
+}
+__device__ __forceinline__ bool head_broken8(const Sync8* sy, unsigned* status) {
+  const bool broken = __hip_atomic_load(&sy->broken, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != 0;
+  if (broken && threadIdx.x == 0 && status != nullptr) atomicAdd(status, 1u);
+  return broken;
+}
 
 // "lane-indexed" arrays hold, for every lane of the producer, the bytes the same lane of a consumer loads:
 // accumulator-layout registers (column lane%16, rows 4*(lane/16)..+3) packed to bf16, hi pair then lo pair.
@@ -263,12 +295,14 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
 }
 
 // ---------------------------------------------------------------------------------------------------- consumer
-// Wave q holds two copies of its share of G as 16x16 accumulator tiles, lane (n = lane%16, g = lane/16):
-//   G1[vt][i] = G[key 16q + n][value 16*vt + 4g + i]     (rows of its keys; B operand of contractions over values)
-//   G2[kt][i] = G[key 16*kt + 4g + i][value 16q + n]     (columns of its values; B operand of contractions over keys)
+// Two kinds of consumer wave, each with its share of G as 16x16 accumulator tiles, lane (n = lane%16, g = lane/16):
+//   key wave q:   G[vt][i] = G[key 16q + n][value 16*vt + 4g + i]   (rows of its keys; B operand of contractions
+//                 over values): gk, gw and the cotangent of the input state
+//   value wave q: G[kt][i] = G[key 16*kt + 4g + i][value 16q + n]   (columns of its values; B operand of contractions
+//                 over keys): gv
 struct Consumer {
-  f32x4_t G1[4], G2[4];
-  float carry;         // running sum of the decay-gradient recursion, per key (same in the four lanes of a key)
+  f32x4_t G[4];
+  float carry;         // key waves: running sum of the decay-gradient recursion, per key (same in a key's four lanes)
   int q, lane;
 };
 
@@ -335,54 +369,40 @@ __device__ __forceinline__ void split_tiles(const f32x4_t (&G)[4], u32x4_t (&Gh)
   }
 }
 
-__device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ slot, const SnapSlot* __restrict__ snapslot,
-                                        const Wkv6Args& A, int64_t b, int64_t h, int nvalid, bool is_snap,
-                                        const Pre& pre, Pre& pre_next, const Cursor& cu, const Cursor& cu_next,
-                                        bool has_next) {
+// ---- key wave: E_t (G_t v_t) per (token, key), the decay-gradient recursion, gk and gw
+__device__ __forceinline__ void consume_keys(Consumer& C, const Slot* __restrict__ slot, const SnapSlot* __restrict__ snapslot,
+                                             const Wkv6Args& A, int64_t b, int64_t h, int nvalid, bool is_snap,
+                                             const Pre& pre, Pre& pre_next, const Cursor& cu, const Cursor& cu_next,
+                                             bool has_next) {
   const int lane = C.lane, n = lane & 15, g = lane >> 4, q = C.q;
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
   const u32x4_t rq = *reinterpret_cast<const u32x4_t*>(&slot->RQ[q][lane]);   // B operand: rq of tokens 4g.., hi | lo
-  const uint2 dq = slot->DYt[q][lane];
-  const u32x4_t dyq = {dq.x, dq.y, dq.x, dq.y};                                // B operand: dy of tokens 4g.., twice
   const bool keep_end = slot->keep_end != 0;
   const uint32_t resets = (uint32_t)slot->resets;
-  // the cotangent of the chunk-end state, decayed over the chunk: per key
-  {
+  {  // the cotangent of the chunk-end state, decayed over the chunk: per key = per lane
     const float gm = slot->gamma[16 * q + n];
 #pragma unroll
-    for (int vt = 0; vt < 4; ++vt) { C.G1[vt][0] *= gm; C.G1[vt][1] *= gm; C.G1[vt][2] *= gm; C.G1[vt][3] *= gm; }
-#pragma unroll
-    for (int kt = 0; kt < 4; ++kt) {
-      const float4 g4 = *reinterpret_cast<const float4*>(&slot->gamma[16 * kt + 4 * g]);
-      C.G2[kt][0] *= g4.x; C.G2[kt][1] *= g4.y; C.G2[kt][2] *= g4.z; C.G2[kt][3] *= g4.w;
-    }
+    for (int vt = 0; vt < 4; ++vt) { C.G[vt][0] *= gm; C.G[vt][1] *= gm; C.G[vt][2] *= gm; C.G[vt][3] *= gm; }
   }
-  u32x4_t G1h[2], G1l[2], G2h[2], G2l[2];
-  split_tiles(C.G1, G1h, G1l);
-  split_tiles(C.G2, G2h, G2l);
-  f32x4_t PK = zero4, PK2 = zero4;   // [token 4g+i][key 16q+n]:   E_t . (G_t v_t)
-  f32x4_t PV = zero4, PV2 = zero4;   // [token 4g+i][value 16q+n]: G_t^T k_t
+  u32x4_t Gh[2], Gl[2];
+  split_tiles(C.G, Gh, Gl);
+  f32x4_t PK = zero4, PK2 = zero4;   // [token 4g+i][key 16q+n]: E_t . (G_t v_t)
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const u32x4_t vv = *reinterpret_cast<const u32x4_t*>(&slot->V[n][32 * j + 8 * g]);
-    const u32x4_t kh = *reinterpret_cast<const u32x4_t*>(&slot->KH[0][n][32 * j + 8 * g]);
-    const u32x4_t kl = *reinterpret_cast<const u32x4_t*>(&slot->KH[1][n][32 * j + 8 * g]);
-    PK = mfma(vv, G1h[j], PK); PV = mfma(kh, G2h[j], PV);
-    PK2 = mfma(vv, G1l[j], PK2); PV2 = mfma(kh, G2l[j], PV2);
-    PV = mfma(kl, G2h[j], PV);
+    PK = mfma(vv, Gh[j], PK);
+    PK2 = mfma(vv, Gl[j], PK2);
   }
   {
     const u32x4_t n1 = *reinterpret_cast<const u32x4_t*>(&slot->N1[lane]);
-    const u32x4_t n2 = *reinterpret_cast<const u32x4_t*>(&slot->N2[lane]);
     const u32x4_t n1hh = {n1[0], n1[1], n1[0], n1[1]}, n1l0 = {n1[2], n1[3], 0u, 0u}, rq0 = {rq[0], rq[1], 0u, 0u};
     PK = mfma(n1hh, rq, PK);                         // N1_hi (rq_hi + rq_lo)
     PK2 = mfma(n1l0, rq0, PK2);                      // N1_lo rq_hi
-    PV2 = mfma(n2, dyq, PV2);                        // (N2_hi + N2_lo) dy
   }
   // a reset inside the chunk cuts the cotangent of later chunks off from the chunk start
   if (!keep_end) {
 #pragma unroll
-    for (int x = 0; x < 4; ++x) { C.G1[x] = zero4; C.G2[x] = zero4; }
+    for (int x = 0; x < 4; ++x) C.G[x] = zero4;
   }
   // the cotangent of the returned state enters at token length-1 (one chunk per sequence)
   float eI = 0.f;
@@ -392,51 +412,29 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
     eI = A.eI[((size_t)b * A.H + h) * 64 + 16 * q + n];
     const bool keep = slot->keep_snap != 0;
     const float sg1 = snapslot->gamma[16 * q + n];
-    f32x4_t T1[4], T2[4];
+    f32x4_t T1[4];
 #pragma unroll
     for (int vt = 0; vt < 4; ++vt) {
       T1[vt] = load_state4(A.gs_out, A.st_f32, state_el(A, b, h, 16 * q + n, 16 * vt + 4 * g)) * sg1;
-      if (keep) C.G1[vt] += T1[vt];
+      if (keep) C.G[vt] += T1[vt];
     }
-#pragma unroll
-    for (int kt = 0; kt < 4; ++kt) {
-      const float4 sg = *reinterpret_cast<const float4*>(&snapslot->gamma[16 * kt + 4 * g]);
-      const float s4[4] = {sg.x, sg.y, sg.z, sg.w};
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-        T2[kt][i] = ld_state_el(A.gs_out, A.st_f32, state_el(A, b, h, 16 * kt + 4 * g + i, 16 * q + n)) * s4[i];
-      if (keep) C.G2[kt] += T2[kt];
-    }
-    u32x4_t T1h[2], T1l[2], T2h[2], T2l[2];
+    u32x4_t T1h[2], T1l[2];
     split_tiles(T1, T1h, T1l);
-    split_tiles(T2, T2h, T2l);
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
       const u32x4_t vv = *reinterpret_cast<const u32x4_t*>(&snapslot->V[n][32 * j + 8 * g]);
-      const u32x4_t kh = *reinterpret_cast<const u32x4_t*>(&snapslot->KH[0][n][32 * j + 8 * g]);
-      const u32x4_t kl = *reinterpret_cast<const u32x4_t*>(&snapslot->KH[1][n][32 * j + 8 * g]);
-      PK = mfma(vv, T1h[j], PK); PV = mfma(kh, T2h[j], PV);
-      PK2 = mfma(vv, T1l[j], PK2); PV2 = mfma(kh, T2l[j], PV2);
-      PV = mfma(kl, T2h[j], PV);
+      PK = mfma(vv, T1h[j], PK);
+      PK2 = mfma(vv, T1l[j], PK2);
     }
   }
-  // cotangent update, both copies: G <- Gh + sum_s rq_s dy_s^T over the tokens before the first reset
+  // cotangent update: G <- Gh + sum_s rq_s dy_s^T over the tokens before the first reset
 #pragma unroll
   for (int vt = 0; vt < 4; ++vt) {
     const uint2 dd = slot->DYtU[vt][lane];
     const u32x4_t A1 = {dd.x, dd.y, dd.x, dd.y};               // rows = values of tile vt, k-slots = dy of tokens, twice
-    C.G1[vt] = mfma(A1, rq, C.G1[vt]);
+    C.G[vt] = mfma(A1, rq, C.G[vt]);
   }
-  {
-    const uint2 du = slot->DYtU[q][lane];
-    const u32x4_t dyu = {du.x, du.y, du.x, du.y};
-#pragma unroll
-    for (int kt = 0; kt < 4; ++kt) {
-      const u32x4_t ra = *reinterpret_cast<const u32x4_t*>(&slot->RQ[kt][lane]);   // rows = keys of tile kt, hi | lo
-      C.G2[kt] = mfma(ra, dyu, C.G2[kt]);
-    }
-  }
-  // per-token results: register i is token 4g+i, lanes n = 16 consecutive keys (gk, gw) or values (gv)
+  // per-token results: register i is token 4g+i, lanes n = 16 consecutive keys
   float gvk[4], z[4], cy[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -461,12 +459,11 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
     }
     C.carry = cin;
   }
-  uint16_t ok[4], ov[4], ow[4];
+  uint16_t ok[4], ow[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int tok = 4 * g + i;
     ok[i] = f32_to_bf16(slot->RUC[tok][16 * q + n] + gvk[i]);
-    ov[i] = f32_to_bf16(slot->DYR[tok][16 * q + n] + PV[i] + PV2[i]);
     ow[i] = f32_to_bf16(((resets >> tok) & 1u) ? 0.f : cy[i] - pre.er[i]);
   }
   // The next chunk's per-token scalars are requested after the last read of this chunk's (into a second set of
@@ -481,7 +478,6 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
   auto put = [&](int i, bool full) {
     if (full || 4 * g + i < nvalid) {
       *reinterpret_cast<uint16_t*>(cu.gk + lo * 2 + i * cu.tok_bytes) = ok[i];
-      *reinterpret_cast<uint16_t*>(cu.gv + lo * 2 + i * cu.tok_bytes) = ov[i];
       *reinterpret_cast<uint16_t*>(cu.gw + lo * 2 + i * cu.tok_bytes) = ow[i];
     }
   };
@@ -495,14 +491,97 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
   }
 }
 
+// ---- value wave: G_t^T k_t per (token, value) and gv
+__device__ __forceinline__ void consume_values(Consumer& C, const Slot* __restrict__ slot, const SnapSlot* __restrict__ snapslot,
+                                               const Wkv6Args& A, int64_t b, int64_t h, int nvalid, bool is_snap,
+                                               const Cursor& cu) {
+  const int lane = C.lane, n = lane & 15, g = lane >> 4, q = C.q;
+  const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+  const uint2 dq = slot->DYt[q][lane];
+  const u32x4_t dyq = {dq.x, dq.y, dq.x, dq.y};                                // B operand: dy of tokens 4g.., twice
+  const bool keep_end = slot->keep_end != 0;
+#pragma unroll
+  for (int kt = 0; kt < 4; ++kt) {   // the cotangent of the chunk-end state, decayed over the chunk: per key = per register
+    const float4 g4 = *reinterpret_cast<const float4*>(&slot->gamma[16 * kt + 4 * g]);
+    C.G[kt][0] *= g4.x; C.G[kt][1] *= g4.y; C.G[kt][2] *= g4.z; C.G[kt][3] *= g4.w;
+  }
+  u32x4_t Gh[2], Gl[2];
+  split_tiles(C.G, Gh, Gl);
+  f32x4_t PV = zero4, PV2 = zero4;   // [token 4g+i][value 16q+n]: G_t^T k_t
+#pragma unroll
+  for (int j = 0; j < 2; ++j) {
+    const u32x4_t kh = *reinterpret_cast<const u32x4_t*>(&slot->KH[0][n][32 * j + 8 * g]);
+    const u32x4_t kl = *reinterpret_cast<const u32x4_t*>(&slot->KH[1][n][32 * j + 8 * g]);
+    PV = mfma(kh, Gh[j], PV);
+    PV2 = mfma(kh, Gl[j], PV2);
+    PV = mfma(kl, Gh[j], PV);
+  }
+  {
+    const u32x4_t n2 = *reinterpret_cast<const u32x4_t*>(&slot->N2[lane]);
+    PV2 = mfma(n2, dyq, PV2);                        // (N2_hi + N2_lo) dy
+  }
+  if (!keep_end) {
+#pragma unroll
+    for (int x = 0; x < 4; ++x) C.G[x] = zero4;
+  }
+  if (is_snap) {
+    const bool keep = slot->keep_snap != 0;
+    f32x4_t T2[4];
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+      const float4 sg = *reinterpret_cast<const float4*>(&snapslot->gamma[16 * kt + 4 * g]);
+      const float s4[4] = {sg.x, sg.y, sg.z, sg.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        T2[kt][i] = ld_state_el(A.gs_out, A.st_f32, state_el(A, b, h, 16 * kt + 4 * g + i, 16 * q + n)) * s4[i];
+      if (keep) C.G[kt] += T2[kt];
+    }
+    u32x4_t T2h[2], T2l[2];
+    split_tiles(T2, T2h, T2l);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const u32x4_t kh = *reinterpret_cast<const u32x4_t*>(&snapslot->KH[0][n][32 * j + 8 * g]);
+      const u32x4_t kl = *reinterpret_cast<const u32x4_t*>(&snapslot->KH[1][n][32 * j + 8 * g]);
+      PV = mfma(kh, T2h[j], PV);
+      PV2 = mfma(kh, T2l[j], PV2);
+      PV = mfma(kl, T2h[j], PV);
+    }
+  }
+  {
+    const uint2 du = slot->DYtU[q][lane];
+    const u32x4_t dyu = {du.x, du.y, du.x, du.y};
+#pragma unroll
+    for (int kt = 0; kt < 4; ++kt) {
+      const u32x4_t ra = *reinterpret_cast<const u32x4_t*>(&slot->RQ[kt][lane]);   // rows = keys of tile kt, hi | lo
+      C.G[kt] = mfma(ra, dyu, C.G[kt]);
+    }
+  }
+  uint16_t ov[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) ov[i] = f32_to_bf16(slot->DYR[4 * g + i][16 * q + n] + PV[i] + PV2[i]);
+  const size_t lo = (size_t)cu.voff;
+  auto put = [&](int i, bool full) {
+    if (full || 4 * g + i < nvalid) *reinterpret_cast<uint16_t*>(cu.gv + lo * 2 + i * cu.tok_bytes) = ov[i];
+  };
+  if (nvalid == CK) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) put(i, true);
+  } else {
+    rare_path();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) put(i, false);
+  }
+}
+
 }  // namespace
 
-// Step j handles chunk nch-1-j in slot j % RING; hand-shake as in the forward kernels.
-__global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv6_chunk_bwd_r_kernel(Wkv6Args A) {
+// Step j handles chunk nch-1-j in slot j % RING; hand-shake as in the forward kernels.  Waves 0-3 are the key waves,
+// 4-7 the value waves, the rest producers: every SIMD runs one wave of each kind.
+__global__ __launch_bounds__(64 * (NCONS_R + NPROD)) void wkv6_chunk_bwd_r_kernel(Wkv6Args A) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   Slot* slots = reinterpret_cast<Slot*>(smem_raw);
   SnapSlot* snapslot = reinterpret_cast<SnapSlot*>(smem_raw + RING * sizeof(Slot));
-  Sync* sy = reinterpret_cast<Sync*>(smem_raw + RING * sizeof(Slot) + sizeof(SnapSlot));
+  Sync8* sy = reinterpret_cast<Sync8*>(smem_raw + RING * sizeof(Slot) + sizeof(SnapSlot));
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   const int64_t b = blockIdx.x / A.H, h = blockIdx.x % A.H;
@@ -511,19 +590,20 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv6_chunk_bwd_r_kernel(
   const int nch = (int)((A.T + CK - 1) / CK);
   const bool q2drop = (A.flags & 1u) && L < A.T && A.ns != nullptr && A.ns[b * A.T + L] != 0;
   const bool inject = A.gs_out != nullptr && !q2drop;   // a cotangent of the returned state exists
-  if (threadIdx.x < sizeof(Sync) / sizeof(int)) reinterpret_cast<int*>(sy)[threadIdx.x] = 0;
+  if (threadIdx.x < sizeof(Sync8) / sizeof(int)) reinterpret_cast<int*>(sy)[threadIdx.x] = 0;
   __syncthreads();
 
-  if (wave < NCONS) {
+  if (wave < NCONS_R) {
     __builtin_amdgcn_s_setprio(3);
+    const bool keys = wave < 4;
     Consumer C;
-    C.q = wave;
+    C.q = wave & 3;
     C.lane = lane;
     C.carry = 0.f;
     const int n = lane & 15, g = lane >> 4;
     const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int x = 0; x < 4; ++x) { C.G1[x] = zero4; C.G2[x] = zero4; }
+    for (int x = 0; x < 4; ++x) C.G[x] = zero4;
     Cursor cu;
     cu.tok_bytes = (size_t)A.H * 64 * 2;
     const size_t el0 = (((size_t)b * A.T + (size_t)(nch - 1) * CK) * A.H + h) * 64;
@@ -532,39 +612,51 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv6_chunk_bwd_r_kernel(
     cu.gk = reinterpret_cast<char*>(A.gk) + el0 * 2;
     cu.gv = reinterpret_cast<char*>(A.gv) + el0 * 2;
     cu.gw = reinterpret_cast<char*>(A.gw) + el0 * 2;
-    cu.voff = (uint32_t)((4 * g) * (int)A.H * 64 + 16 * wave + n);
+    cu.voff = (uint32_t)((4 * g) * (int)A.H * 64 + 16 * C.q + n);
     const int csnap = (L >= 1 && inject) ? (int)((L - 1) / CK) : -1;
     const int tail = (A.T % CK == 0) ? CK : (int)(A.T % CK);
-    Pre pre_a, pre_b;
-    if (nch > 0) prefetch(pre_a, cu, tail, g);
-    auto step = [&](int j, const Pre& pre, Pre& pre_next) -> bool {
-      const int c = nch - 1 - j;
-      const int nvalid = (j == 0) ? tail : CK;
-      const int si = j % RING;
-      Cursor nxt = cu;
-      step_back(nxt);
-      if (!wait_ready(sy, si, j + 1)) return false;
-      consume(C, &slots[si], snapslot, A, b, h, nvalid, c == csnap, pre, pre_next, cu, nxt, j + 1 < nch);
-      cu = nxt;
-      if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
-      return true;
-    };
-    for (int j = 0; j < nch; j += 2) {      // two steps per turn: the prefetch registers alternate
-      if (!step(j, pre_a, pre_b)) break;
-      if (j + 1 < nch && !step(j + 1, pre_b, pre_a)) break;
-    }
-    // cotangent of the input state; with length == 0 the returned state is the input state itself
-    const bool pass = L == 0 && inject;
+    if (keys) {
+      Pre pre_a, pre_b;
+      if (nch > 0) prefetch(pre_a, cu, tail, g);
+      auto step = [&](int j, const Pre& pre, Pre& pre_next) -> bool {
+        const int c = nch - 1 - j;
+        const int nvalid = (j == 0) ? tail : CK;
+        const int si = j % RING;
+        Cursor nxt = cu;
+        step_back(nxt);
+        if (!wait_ready8(sy, si, j + 1)) return false;
+        consume_keys(C, &slots[si], snapslot, A, b, h, nvalid, c == csnap, pre, pre_next, cu, nxt, j + 1 < nch);
+        cu = nxt;
+        if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+        return true;
+      };
+      for (int j = 0; j < nch; j += 2) {      // two steps per turn: the prefetch registers alternate
+        if (!step(j, pre_a, pre_b)) break;
+        if (j + 1 < nch && !step(j + 1, pre_b, pre_a)) break;
+      }
+      // cotangent of the input state; with length == 0 the returned state is the input state itself
+      const bool pass = L == 0 && inject;
 #pragma unroll
-    for (int vt = 0; vt < 4; ++vt) {
-      const size_t off = state_el(A, b, h, 16 * wave + n, 16 * vt + 4 * g);
-      f32x4_t gsv = C.G1[vt];
-      if (pass) gsv += load_state4(A.gs_out, A.st_f32, off);
-      if (A.st_f32) *reinterpret_cast<float4*>(reinterpret_cast<float*>(A.gs) + off) = make_float4(gsv[0], gsv[1], gsv[2], gsv[3]);
-      else *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(A.gs) + off) = make_uint2(pack_rn(gsv[0], gsv[1]), pack_rn(gsv[2], gsv[3]));
+      for (int vt = 0; vt < 4; ++vt) {
+        const size_t off = state_el(A, b, h, 16 * C.q + n, 16 * vt + 4 * g);
+        f32x4_t gsv = C.G[vt];
+        if (pass) gsv += load_state4(A.gs_out, A.st_f32, off);
+        if (A.st_f32) *reinterpret_cast<float4*>(reinterpret_cast<float*>(A.gs) + off) = make_float4(gsv[0], gsv[1], gsv[2], gsv[3]);
+        else *reinterpret_cast<uint2*>(reinterpret_cast<uint16_t*>(A.gs) + off) = make_uint2(pack_rn(gsv[0], gsv[1]), pack_rn(gsv[2], gsv[3]));
+      }
+    } else {
+      for (int j = 0; j < nch; ++j) {
+        const int c = nch - 1 - j;
+        const int nvalid = (j == 0) ? tail : CK;
+        const int si = j % RING;
+        if (!wait_ready8(sy, si, j + 1)) break;
+        consume_values(C, &slots[si], snapslot, A, b, h, nvalid, c == csnap, cu);
+        step_back(cu);
+        if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+      }
     }
   } else {
-    const int p = wave - NCONS;
+    const int p = wave - NCONS_R;
     Producer P;
     P.lane = lane;
     make_sel(P.sel, lane);
@@ -582,7 +674,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv6_chunk_bwd_r_kernel(
       if (!inject) F.snap = -1;
       const int si = j % RING;
       Slot* slot = &slots[si];
-      if (j >= RING && !wait_consumed(sy, si, j - RING + 1, lane)) break;
+      if (j >= RING && !wait_consumed8(sy, si, j - RING + 1, lane)) break;
       produce(P, raw, F, slot, snapslot);
       if (j + NPROD < nch) load_raw(raw, A, b, h, (int64_t)(c - NPROD) * CK, lane);
       if ((A.flags & FLAG_DROP_PUBLISH) && j + 1 == nch) break;
@@ -590,7 +682,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv6_chunk_bwd_r_kernel(
     }
   }
   __syncthreads();
-  if (head_broken(sy, A.status)) {
+  if (head_broken8(sy, A.status)) {
     poison_token_rows(A.gk, 2, b, h, A.T, A.H);
     poison_token_rows(A.gv, 2, b, h, A.T, A.H);
     poison_token_rows(A.gw, 2, b, h, A.T, A.H);
@@ -599,11 +691,11 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv6_chunk_bwd_r_kernel(
 }
 
 hipError_t launch_wkv6_chunk_bwd_r(const Wkv6Args& A, hipStream_t stream) {
-  const size_t smem = RING * sizeof(Slot) + sizeof(SnapSlot) + sizeof(Sync);
+  const size_t smem = RING * sizeof(Slot) + sizeof(SnapSlot) + sizeof(Sync8);
   static LdsAttrOnce once;
   const hipError_t attr = allow_dynamic_lds(once, reinterpret_cast<const void*>(wkv6_chunk_bwd_r_kernel), smem);
   if (attr != hipSuccess) return attr;
-  hipLaunchKernelGGL(wkv6_chunk_bwd_r_kernel, dim3((unsigned)(A.B * A.H)), dim3(64 * (NCONS + NPROD)), smem, stream, A);
+  hipLaunchKernelGGL(wkv6_chunk_bwd_r_kernel, dim3((unsigned)(A.B * A.H)), dim3(64 * (NCONS_R + NPROD)), smem, stream, A);
   return hipGetLastError();
 }
 
