@@ -88,6 +88,20 @@ int hiprwkv_wkv7_fwd(hiprwkv_stream stream, int io_dtype, int state_dtype,
                      const uint32_t* length, const uint8_t* new_starts,
                      void* out, void* sa, void* new_s, unsigned flags);
 
+/* A decode step (T <= HIPRWKV_SMALL_T tokens per sequence) on a state that lives inside the packed model state of the
+ * reference: there a sequence's state is (L, 2+N, C) and layer l's rows 2.. are the (H,N,N) WKV state, flat
+ * (rwkv7.py:176-180 default_state, :254-260 the slice and reshape around inner_loop), so with a batch axis in front
+ * the states of consecutive sequences are H*N*N contiguous elements each, L*(2+N)*C elements apart.  `s` and `new_s`
+ * point at the first sequence's state, `*_batch_stride` is that distance in elements (>= H*N*N, a multiple of 16
+ * bytes); everything else is as in hiprwkv_wkv7_fwd without `sa`.  Every element of a state is read once, before
+ * anything is written, by the thread that writes it: `new_s` may be `s` (same stride) for an update in place. */
+int hiprwkv_wkv7_step(hiprwkv_stream stream, int io_dtype, int state_dtype,
+                      int64_t B, int64_t T, int64_t H, int64_t N,
+                      const void* w, const void* r, const void* k, const void* v,
+                      const void* a, const void* b, const void* s, int64_t s_batch_stride,
+                      const uint32_t* length, const uint8_t* new_starts,
+                      void* out, void* new_s, int64_t new_s_batch_stride, unsigned flags);
+
 /* Bytes of scratch hiprwkv_wkv7_bwd needs for this shape. */
 size_t hiprwkv_wkv7_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t N);
 

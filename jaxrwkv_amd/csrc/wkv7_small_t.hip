@@ -36,10 +36,16 @@ __global__ __launch_bounds__(256) void wkv7_small_t_kernel(Wkv7Args A) {
   const uint8_t* ns = A.ns ? A.ns + b * A.T : nullptr;
   // the returned state is the reset state there (associative-scan rule)
   const bool q2drop = compat && L < A.T && ns != nullptr && ns[L] != 0;
-  const size_t sel = (((size_t)b * A.H + h) * 64 + i) * 64 + c0;
+  // a sequence's state is H*64*64 contiguous elements; consecutive sequences may lie further apart (a layer's rows of
+  // a packed model state).  Every thread reads its 16 elements once, up front, and writes them once: s and new_s may
+  // be the same memory.
+  const size_t in_head = ((size_t)h * 64 + i) * 64 + c0;
+  const size_t dense = (size_t)A.H * 4096;
+  const size_t sel = (size_t)b * (A.s_bstride ? (size_t)A.s_bstride : dense) + in_head;
+  const size_t sel_out = (size_t)b * (A.new_s_bstride ? (size_t)A.new_s_bstride : dense) + in_head;
   float S[16];
   ld16<ST>(A.s, sel, S);
-  if (L == 0) st16<ST>(A.new_s, sel, S, q2drop);   // rwkv7.py:203
+  if (L == 0) st16<ST>(A.new_s, sel_out, S, q2drop);   // rwkv7.py:203
   for (int64_t t = 0; t < A.T; ++t) {
     const size_t tel = (((size_t)b * A.T + t) * A.H + h) * 64;
     float w[16], r[16], k[16], a[16], bb[16];
@@ -74,7 +80,7 @@ __global__ __launch_bounds__(256) void wkv7_small_t_kernel(Wkv7Args A) {
         else reinterpret_cast<_Float16*>(A.sa)[tel + i] = (_Float16)sa;
       }
     }
-    if (t == L - 1) st16<ST>(A.new_s, sel, S, q2drop);
+    if (t == L - 1) st16<ST>(A.new_s, sel_out, S, q2drop);
   }
 }
 

@@ -24,6 +24,9 @@ struct Wkv7Args {
   void *gw, *gr, *gk, *gv, *ga, *gb, *gs;
   float *dsa, *e2, *e3;  // workspace, (B,T,H,64) fp32 each (the chunked sweeps keep e3_t + e2_{t+1} in e2, e3 unused)
   unsigned* status;      // device word counting workgroups whose hand-shake gave up (may be null)
+  // Elements between the states of consecutive sequences in `s` / `new_s`; 0 = dense (H*64*64).  Honoured by the
+  // small-T kernel only (states read and written inside a packed model state).
+  int64_t s_bstride, new_s_bstride;
 };
 
 // Wkv6Args::flags bit: w is (H,64), shared by every token and sequence (HIPRWKV_W_PER_HEAD)

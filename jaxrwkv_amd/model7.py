@@ -142,8 +142,11 @@ class RWKV7:
         return k @ ffn["value"]["weight"].T, x[torch.arange(x.shape[0], device=x.device), last_idx]
 
     @classmethod
-    def time_mixing_seq(cls, x, shift_row, wkv_state, v_first, att, length, last_idx, new_starts, layer_id):
-        """rwkv7.py:223-267.  wkv_state (B, N, C) is the layer's rows 2.. of the model state."""
+    def time_mixing_seq(cls, x, shift_row, wkv_state, v_first, att, length, last_idx, new_starts, layer_id,
+                        wkv_out=None):
+        """rwkv7.py:223-267.  wkv_state (B, N, C) is the layer's rows 2.. of the model state.  With ``wkv_out`` (the
+        same rows of the new model state; decode steps without autograd) the recurrence reads and writes the two views
+        in place and the third result is None."""
         B, T, C = x.shape
         H, N = att["r_k"].shape
         sx = cls._shift(x, shift_row, new_starts)
@@ -159,7 +162,6 @@ class RWKV7:
         a = torch.sigmoid(att["a0"] + (xa @ att["a1"]) @ att["a2"])
         g = torch.sigmoid(xg @ att["g1"]) @ att["g2"]
         new_shift = x[torch.arange(B, device=x.device), last_idx]
-        s = wkv_state.reshape(B, H, N, N)
         fused = cls.fuse_mix
         rh, wh, vh = (t.reshape(B, T, H, N) for t in (r, w, v))
         if fused:
@@ -170,7 +172,11 @@ class RWKV7:
             kk = kk.reshape(B, T, C)
             k = k * (1 + (a - 1) * att["k_a"])
             kh, ah, bh = (t.reshape(B, T, H, N) for t in (k, -kk, kk * a))
-        s_new, out = cls.inner.inner_loop(rh, wh, kh, vh, ah, bh, s, length, new_starts)
+        if wkv_out is not None:
+            s_new, out = None, cls.inner.step_packed(rh, wh, kh, vh, ah, bh, wkv_state, wkv_out, length, new_starts)
+        else:
+            s_new, out = cls.inner.inner_loop(rh, wh, kh, vh, ah, bh, wkv_state.reshape(B, H, N, N), length, new_starts)
+            s_new = s_new.reshape(B, N, C)
         if fused:
             y = ops.rwkv7_postmix(out, rh, kh, vh, g.reshape(B, T, H, N), att["ln_x"]["weight"], att["ln_x"]["bias"],
                                   att["r_k"], 64e-5).reshape(B, T, C)
@@ -180,7 +186,7 @@ class RWKV7:
             y = y.to(x.dtype).reshape(B, T, C)
             bonus = ((rh * kh * att["r_k"]).sum(-1, keepdim=True) * vh).reshape(B, T, C)
             y = (y + bonus) * g
-        return y @ att["output"]["weight"].T, new_shift, s_new.reshape(B, N, C), v_first
+        return y @ att["output"]["weight"].T, new_shift, s_new, v_first
 
     @classmethod
     def forward(cls, params, tokens, state, length=None, new_starts=None):
@@ -198,17 +204,22 @@ class RWKV7:
         x = layer_norm(x, params["ln0"])
         L = params["blocks"]["att"]["r_k"].shape[0]
         new_state = torch.empty_like(state)
+        # decode steps: the recurrence works on the layers' rows of the two model states directly (no copies of them)
+        packed = (T <= 8 and hasattr(cls.inner, "step_packed")
+                  and not (torch.is_grad_enabled() and (x.requires_grad or state.requires_grad)))
         v_first = x
         for i in range(L):
             blk = layer_of(params["blocks"], i)
             st = state[:, i]
             dx, shift1, wkv, v_first = cls.time_mixing_seq(layer_norm(x, blk["ln1"]), st[:, 1], st[:, 2:], v_first,
-                                                           blk["att"], length, last_idx, new_starts, i)
+                                                           blk["att"], length, last_idx, new_starts, i,
+                                                           new_state[:, i, 2:] if packed else None)
             x = x + dx
             dx, shift0 = cls.channel_mixing_seq(layer_norm(x, blk["ln2"]), st[:, 0], blk["ffn"], last_idx, new_starts)
             x = x + dx
             new_state[:, i, 0] = shift0
             new_state[:, i, 1] = shift1
-            new_state[:, i, 2:] = wkv.to(state.dtype)
+            if not packed:
+                new_state[:, i, 2:] = wkv.to(state.dtype)
         logits = layer_norm(x, params["ln_out"]) @ params["head"]["weight"].T
         return logits, new_state

@@ -87,6 +87,33 @@ def wkv7_fwd(r, w, k, v, a, b, s, length=None, new_starts=None, compat=True, wan
     return new_s, y, sa
 
 
+def _packed_state(t, B, H, N):
+    """(pointer tensor, batch stride in elements) of a state view whose sequences are H*N*N contiguous elements each."""
+    assert t.is_cuda and t.shape[0] == B and t[0].numel() == H * N * N, (t.shape, (B, H, N))
+    assert t[0].is_contiguous(), "a sequence's state must be contiguous"
+    return t, (t.stride(0) if B > 1 else H * N * N)
+
+
+def wkv7_step(r, w, k, v, a, b, s, new_s, length=None, new_starts=None, compat=True):
+    """A decode step (T <= 8) on states inside a packed model state: ``s`` and ``new_s`` are views with a batch axis in
+    front and H*N*N contiguous elements per sequence, e.g. ``state[:, layer, 2:]`` of a ``(B, L, 2+N, C)`` model state
+    (rwkv7.py:176-180, 254-260); ``new_s`` is written in place (it may be ``s``).  Returns y.  No autograd."""
+    lib = _lib.load()
+    io = r.dtype
+    r, w, k, v, a, b = (_dev(x, io) for x in (r, w, k, v, a, b))
+    B, T, H, N = r.shape
+    s, s_stride = _packed_state(s, B, H, N)
+    new_s, ns_stride = _packed_state(new_s, B, H, N)
+    assert s.dtype == new_s.dtype
+    length, new_starts = _length_ns(length, new_starts, B, T, r.device)
+    y = torch.empty_like(r)
+    rc = lib.hiprwkv_wkv7_step(_stream(), _DT[io], _DT[s.dtype], B, T, H, N, _p(w), _p(r), _p(k), _p(v), _p(a), _p(b),
+                               _p(s), s_stride, _p(length), _p(new_starts), _p(y), _p(new_s), ns_stride,
+                               _flags(compat, False, True, 0))
+    _lib.check(rc, "hiprwkv_wkv7_step")
+    return y
+
+
 def wkv7_bwd(r, w, k, v, a, b, s, length, new_starts, gy, sa, gs_out=None, compat=True, force_seq=False,
              debug_flags=0):
     """Cotangents (gr, gw, gk, gv, ga, gb, gs) of ``wkv7_fwd`` for cotangents gy of y and gs_out of new_s.

@@ -34,3 +34,10 @@ class HipRWKV:
         if not batched:
             new_s, y = new_s[0], y[0]
         return new_s, y
+
+    @classmethod
+    def step_packed(cls, r, w, k, v, a, b, s, new_s, length, new_starts):
+        """``inner_loop`` for a few tokens (T <= 8, decode) with the state read from and written to views of the packed
+        model state (``state[:, layer, 2:]``, rwkv7.py:254-260) instead of copies of them; batched, no autograd.
+        Returns ``out``; ``new_s`` is filled in place."""
+        return ops.wkv7_step(r, w, k, v, a, b, s, new_s, length, new_starts, cls.assoc_compat)

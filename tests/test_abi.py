@@ -59,6 +59,13 @@ def test_argument_validation_without_gpu():
     rc = lib.hiprwkv_wkv4_fwd_ckpt(null, 0, 0, 17, 64, *([ok] * 5), null, null, ok, ok, ok, 1 << 20, 0)
     assert rc == -1
     assert lib.hiprwkv_wkv7_bwd_workspace_bytes(2, 16, 2, 64) == 3 * 2 * 16 * 2 * 64 * 4
+    # the decode step on a packed state: at most 8 tokens, batch strides of at least one state and 16-byte multiples
+    step = lambda T, s_stride, o_stride, st=1: lib.hiprwkv_wkv7_step(null, 1, st, 2, T, 2, 64, *([ok] * 7), s_stride, null,
+                                                                   null, ok, ok, o_stride, 0)
+    assert step(9, 8192, 8192) == -1 and b"at most 8" in lib.hiprwkv_last_error()
+    assert step(1, 8191, 8192) == -1 and b"less than" in lib.hiprwkv_last_error()
+    assert step(1, 8192, 8192 + 4) == -1 and b"16 bytes" in lib.hiprwkv_last_error()
+    assert step(1, 8192 + 2, 8192, st=0) == -1 and b"16 bytes" in lib.hiprwkv_last_error()
     assert lib.hiprwkv_wkv6_bwd_workspace_bytes(2, 16, 2, 64) >= 2 * 16 * 2 * 64 * 4
 
 
