@@ -14,7 +14,7 @@ typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
 
 constexpr int CK = 16;            // tokens per chunk
 constexpr int RS = 72;            // row stride (bf16 elements) of the [token][64] LDS arrays: 144 B (16-byte aligned rows)
-constexpr int NCONS = 4;          // consumer waves, one per 16 value rows
+constexpr int NCONS = 4;          // consumer waves, one per 16 value rows (the WKV6 reverse sweep has eight)
 constexpr int SPIN_LIMIT = 1 << 16;   // polls before a waiter gives up (milliseconds; a healthy wait is microseconds)
 constexpr float LOG2E = 1.44269504088896340736f;
 constexpr float MIN_STEP_L2 = -1.0e4f;          // keeps the running sum finite
@@ -26,14 +26,17 @@ constexpr float MIN_CUM_L2 = -80.0f * LOG2E;    // floor of a chunk's total log2
 // workgroup's final barrier every output of that (sequence, head) is overwritten with NaN and the library's
 // failure counter is incremented (finish_head below), so no launch returns stale data unnoticed.
 constexpr int MAX_RING = 16;      // most slots a ring may have
-struct __attribute__((aligned(16))) Sync {
+template <int NC>                 // NC = number of consumer waves
+struct __attribute__((aligned(16))) SyncN {
   int ready[MAX_RING];
-  int consumed[NCONS][MAX_RING];
+  int consumed[NC][MAX_RING];
   int broken;
   int pad[3];
 };
+using Sync = SyncN<NCONS>;
 
-__device__ __forceinline__ bool wait_ready(Sync* sy, int slot, int want) {
+template <int NC>
+__device__ __forceinline__ bool wait_ready(SyncN<NC>* sy, int slot, int want) {
   for (int spin = 0; spin < SPIN_LIMIT; ++spin) {
     if (__hip_atomic_load(&sy->ready[slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) == want) return true;
     __builtin_amdgcn_s_sleep(1);
@@ -41,10 +44,11 @@ __device__ __forceinline__ bool wait_ready(Sync* sy, int slot, int want) {
   __hip_atomic_store(&sy->broken, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   return false;
 }
-__device__ __forceinline__ bool wait_consumed(Sync* sy, int slot, int want, int lane) {
+template <int NC>
+__device__ __forceinline__ bool wait_consumed(SyncN<NC>* sy, int slot, int want, int lane) {
   for (int spin = 0; spin < SPIN_LIMIT; ++spin) {
     int seen = want;
-    if (lane < NCONS) seen = __hip_atomic_load(&sy->consumed[lane][slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (lane < NC) seen = __hip_atomic_load(&sy->consumed[lane][slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
     if (__ballot(seen < want) == 0ull) return true;
     __builtin_amdgcn_s_sleep(1);
   }
@@ -56,20 +60,23 @@ __device__ __forceinline__ bool wait_consumed(Sync* sy, int slot, int want, int 
 // still in use sleeps for hundreds of cycles between polls (every poll costs vector instructions that compete with
 // the consumer on the same SIMD); a consumer tests a flag value that it requested earlier in the chunk, so that the
 // LDS round trip is off its critical path, and only polls if that value was not the wanted one yet.
-__device__ __forceinline__ bool wait_consumed_lazy(Sync* sy, int slot, int want, int lane) {
+template <int NC>
+__device__ __forceinline__ bool wait_consumed_lazy(SyncN<NC>* sy, int slot, int want, int lane) {
   for (int spin = 0; spin < SPIN_LIMIT / 8; ++spin) {
     int seen = want;
-    if (lane < NCONS) seen = __hip_atomic_load(&sy->consumed[lane][slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (lane < NC) seen = __hip_atomic_load(&sy->consumed[lane][slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
     if (__ballot(seen < want) == 0ull) return true;
     __builtin_amdgcn_s_sleep(8);
   }
   __hip_atomic_store(&sy->broken, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   return false;
 }
-__device__ __forceinline__ int peek_ready(const Sync* sy, int slot) {
+template <int NC>
+__device__ __forceinline__ int peek_ready(const SyncN<NC>* sy, int slot) {
   return __hip_atomic_load(&sy->ready[slot], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
 }
-__device__ __forceinline__ bool wait_ready_peeked(Sync* sy, int slot, int want, int peeked) {
+template <int NC>
+__device__ __forceinline__ bool wait_ready_peeked(SyncN<NC>* sy, int slot, int want, int peeked) {
   if (__builtin_amdgcn_readfirstlane(peeked) == want) {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
     return true;
@@ -103,7 +110,8 @@ __device__ __forceinline__ void poison_state(void* base, int f32, int64_t b, int
     reinterpret_cast<uint4*>(p)[i] = make_uint4(nan, nan, nan, nan);
 }
 // After the workgroup's final barrier: did any waiter of this workgroup give up?
-__device__ __forceinline__ bool head_broken(const Sync* sy, unsigned* status) {
+template <int NC>
+__device__ __forceinline__ bool head_broken(const SyncN<NC>* sy, unsigned* status) {
   const bool broken = __hip_atomic_load(&sy->broken, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != 0;
   if (broken && threadIdx.x == 0 && status != nullptr) atomicAdd(status, 1u);
   return broken;

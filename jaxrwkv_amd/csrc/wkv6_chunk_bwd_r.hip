@@ -31,35 +31,7 @@ constexpr int RING = 5;           // slots in flight (a slot is 30 KB)
 constexpr int ES = 68;            // row stride (floats) of the fp32 [token][.] arrays: conflict-free column reads
 constexpr int NCONS_R = 8;        // consumer waves: 0-3 hold G1 (gk, gw, gs), 4-7 hold G2 (gv)
 
-struct __attribute__((aligned(16))) Sync8 {      // the hand-shake words of chunk_common.h for eight consumers
-  int ready[MAX_RING];
-  int consumed[NCONS_R][MAX_RING];
-  int broken;
-  int pad[3];
-};
-__device__ __forceinline__ bool wait_ready8(Sync8* sy, int slot, int want) {
-  for (int spin = 0; spin < SPIN_LIMIT; ++spin) {
-    if (__hip_atomic_load(&sy->ready[slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP) == want) return true;
-    __builtin_amdgcn_s_sleep(1);
-  }
-  __hip_atomic_store(&sy->broken, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-  return false;
-}
-__device__ __forceinline__ bool wait_consumed8(Sync8* sy, int slot, int want, int lane) {
-  for (int spin = 0; spin < SPIN_LIMIT; ++spin) {
-    int seen = want;
-    if (lane < NCONS_R) seen = __hip_atomic_load(&sy->consumed[lane][slot], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_WORKGROUP);
-    if (__ballot(seen < want) == 0ull) return true;
-    __builtin_amdgcn_s_sleep(1);
-  }
-  __hip_atomic_store(&sy->broken, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-  return false;
-}
-__device__ __forceinline__ bool head_broken8(const Sync8* sy, unsigned* status) {
-  const bool broken = __hip_atomic_load(&sy->broken, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP) != 0;
-  if (broken && threadIdx.x == 0 && status != nullptr) atomicAdd(status, 1u);
-  return broken;
-}
+using Sync8 = SyncN<NCONS_R>;     // the hand-shake words for eight consumers
 
 // "lane-indexed" arrays hold, for every lane of the producer, the bytes the same lane of a consumer loads:
 // accumulator-layout registers (column lane%16, rows 4*(lane/16)..+3) packed to bf16, hi pair then lo pair.
@@ -624,7 +596,7 @@ __global__ __launch_bounds__(64 * (NCONS_R + NPROD)) void wkv6_chunk_bwd_r_kerne
         const int si = j % RING;
         Cursor nxt = cu;
         step_back(nxt);
-        if (!wait_ready8(sy, si, j + 1)) return false;
+        if (!wait_ready(sy, si, j + 1)) return false;
         consume_keys(C, &slots[si], snapslot, A, b, h, nvalid, c == csnap, pre, pre_next, cu, nxt, j + 1 < nch);
         cu = nxt;
         if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -649,7 +621,7 @@ __global__ __launch_bounds__(64 * (NCONS_R + NPROD)) void wkv6_chunk_bwd_r_kerne
         const int c = nch - 1 - j;
         const int nvalid = (j == 0) ? tail : CK;
         const int si = j % RING;
-        if (!wait_ready8(sy, si, j + 1)) break;
+        if (!wait_ready(sy, si, j + 1)) break;
         consume_values(C, &slots[si], snapslot, A, b, h, nvalid, c == csnap, cu);
         step_back(cu);
         if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -674,7 +646,7 @@ __global__ __launch_bounds__(64 * (NCONS_R + NPROD)) void wkv6_chunk_bwd_r_kerne
       if (!inject) F.snap = -1;
       const int si = j % RING;
       Slot* slot = &slots[si];
-      if (j >= RING && !wait_consumed8(sy, si, j - RING + 1, lane)) break;
+      if (j >= RING && !wait_consumed(sy, si, j - RING + 1, lane)) break;
       produce(P, raw, F, slot, snapslot);
       if (j + NPROD < nch) load_raw(raw, A, b, h, (int64_t)(c - NPROD) * CK, lane);
       if ((A.flags & FLAG_DROP_PUBLISH) && j + 1 == nch) break;
@@ -682,7 +654,7 @@ __global__ __launch_bounds__(64 * (NCONS_R + NPROD)) void wkv6_chunk_bwd_r_kerne
     }
   }
   __syncthreads();
-  if (head_broken8(sy, A.status)) {
+  if (head_broken(sy, A.status)) {
     poison_token_rows(A.gk, 2, b, h, A.T, A.H);
     poison_token_rows(A.gv, 2, b, h, A.T, A.H);
     poison_token_rows(A.gw, 2, b, h, A.T, A.H);
