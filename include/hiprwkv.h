@@ -191,6 +191,24 @@ int hiprwkv_wkv4_bwd_noalloc(hiprwkv_stream stream, int io_dtype,
                              const uint32_t* length, const uint8_t* new_starts, const void* gs_new,
                              float* gw, float* gu, void* gk, void* gv, void* gs, unsigned flags);
 
+/* ---- RWKV-7 token shift and interpolation ---------------------------------------------------
+ * The head of time_mixing_seq and channel_mixing_seq (rwkv7.py:226-235 and :192-195), which the reference computes in
+ * jnp; no counterpart among its ffi targets:
+ *     sx_t = (new_starts[t] ? 0 : x_{t-1}) - x_t ,  out_i = x + sx . mix_i ,  i < n_out   (6: x_r x_w x_k x_v x_a x_g; 1: x_k)
+ * x and every out_i are (B,T,C) io_dtype; `prev` is the token before t = 0 of every sequence, C elements each,
+ * `prev_batch_stride` elements apart (>= C, a multiple of 16 bytes: the layer's shift row inside the packed model
+ * state, rwkv7.py:254, :284); `mix` and `out` are host arrays of n_out device pointers, mix[i] a (C,) io_dtype
+ * parameter.  C must be a multiple of 8.  new_starts (B,T) bytes or NULL. */
+int hiprwkv_rwkv7_shiftmix(hiprwkv_stream stream, int io_dtype, int64_t B, int64_t T, int64_t C, int n_out,
+                           const void* x, const void* prev, int64_t prev_batch_stride, const uint8_t* new_starts,
+                           const void* const* mix, void* const* out);
+/* Cotangents for cotangents g[i] (B,T,C) of the outputs: dx (B,T,C) and dprev (C elements per sequence,
+ * `dprev_batch_stride` apart) in io_dtype, dmix (n_out, C) fp32, summed over sequences and tokens (zeroed by the call). */
+int hiprwkv_rwkv7_shiftmix_bwd(hiprwkv_stream stream, int io_dtype, int64_t B, int64_t T, int64_t C, int n_out,
+                               const void* x, const void* prev, int64_t prev_batch_stride, const uint8_t* new_starts,
+                               const void* const* mix, const void* const* g, void* dx, void* dprev,
+                               int64_t dprev_batch_stride, float* dmix);
+
 /* ---- RWKV-7 time-mixing stages around the op ------------------------------------------
  * The element-wise work the reference does in jnp on either side of inner_loop (rwkv7.py:248-252, 257 and :263-265),
  * fused into one pass each; it has no counterpart among the reference's ffi targets.  `rows` = number of tokens

@@ -93,7 +93,7 @@ unsigned* status_word() {
 extern "C" {
 
 const char* hiprwkv_last_error(void) { return g_err; }
-int hiprwkv_version(void) { return 103; }
+int hiprwkv_version(void) { return 104; }
 
 int hiprwkv_handshake_failures(hiprwkv_stream stream, unsigned* count) {
   if (count == nullptr) return fail(HIPRWKV_EINVAL, "handshake_failures: null count pointer");
@@ -393,6 +393,62 @@ int hiprwkv_wkv4_bwd_noalloc(hiprwkv_stream stream, int io_dtype, int64_t B, int
   if (ws == nullptr) return HIPRWKV_ELAUNCH;
   return hiprwkv_wkv4_bwd(stream, io_dtype, B, T, C, w, u, k, v, gy, s, length, new_starts, gs_new, gw, gu, gk, gv,
                           gs, ws, SCRATCH_BYTES, flags);
+}
+
+namespace {
+int check_shiftmix(const char* op, int io_dtype, int64_t B, int64_t T, int64_t C, int n_out, const void* x,
+                   const void* prev, int64_t prev_bstride, const void* const* mix, const void* const* per_out) {
+  if (!dtype_ok(io_dtype)) return fail(HIPRWKV_EINVAL, "%s: dtype must be HIPRWKV_F32 or HIPRWKV_BF16", op);
+  if (B <= 0 || T <= 0 || C <= 0 || C % 8 != 0) return fail(HIPRWKV_EINVAL, "%s: B, T must be positive and C a positive multiple of 8", op);
+  if (B * T * (C / 8) > 0x7fffffffLL * 256) return fail(HIPRWKV_EINVAL, "%s: too many elements for one launch", op);
+  if (n_out != 1 && n_out != 6) return fail(HIPRWKV_EINVAL, "%s: n_out must be 1 (channel mixing) or 6 (time mixing)", op);
+  if (mix == nullptr || per_out == nullptr) return fail(HIPRWKV_EINVAL, "%s: null pointer array", op);
+  const int64_t elem = io_dtype == HIPRWKV_F32 ? 4 : 2;
+  if (prev_bstride < C || (prev_bstride * elem) % 16 != 0)
+    return fail(HIPRWKV_EINVAL, "%s: the batch stride of the shift row must be at least C and a multiple of 16 bytes", op);
+  const void* req[] = {x, prev};
+  for (const void* p : req) {
+    if (p == nullptr) return fail(HIPRWKV_EINVAL, "%s: null tensor pointer", op);
+    if (!aligned16(p)) return fail(HIPRWKV_EINVAL, "%s: tensor pointers must be 16-byte aligned", op);
+  }
+  for (int i = 0; i < n_out; ++i) {
+    if (mix[i] == nullptr || per_out[i] == nullptr) return fail(HIPRWKV_EINVAL, "%s: null tensor pointer", op);
+    if (!aligned16(mix[i]) || !aligned16(per_out[i])) return fail(HIPRWKV_EINVAL, "%s: tensor pointers must be 16-byte aligned", op);
+  }
+  return HIPRWKV_OK;
+}
+}  // namespace
+
+int hiprwkv_rwkv7_shiftmix(hiprwkv_stream stream, int io_dtype, int64_t B, int64_t T, int64_t C, int n_out, const void* x,
+                           const void* prev, int64_t prev_batch_stride, const uint8_t* new_starts,
+                           const void* const* mix, void* const* out) {
+  int rc = check_shiftmix("rwkv7_shiftmix", io_dtype, B, T, C, n_out, x, prev, prev_batch_stride, mix,
+                          const_cast<const void* const*>(out));
+  if (rc) return rc;
+  hipError_t e = launch_rwkv7_shiftmix(io_dtype == HIPRWKV_F32, B, T, C, n_out, x, prev, prev_batch_stride, new_starts,
+                                       mix, out, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "rwkv7_shiftmix: %s", hipGetErrorString(e));
+  return HIPRWKV_OK;
+}
+
+int hiprwkv_rwkv7_shiftmix_bwd(hiprwkv_stream stream, int io_dtype, int64_t B, int64_t T, int64_t C, int n_out,
+                               const void* x, const void* prev, int64_t prev_batch_stride, const uint8_t* new_starts,
+                               const void* const* mix, const void* const* g, void* dx, void* dprev,
+                               int64_t dprev_batch_stride, float* dmix) {
+  int rc = check_shiftmix("rwkv7_shiftmix_bwd", io_dtype, B, T, C, n_out, x, prev, prev_batch_stride, mix, g);
+  if (rc) return rc;
+  const void* req[] = {dx, dprev, dmix};
+  for (const void* p : req) {
+    if (p == nullptr) return fail(HIPRWKV_EINVAL, "rwkv7_shiftmix_bwd: null tensor pointer");
+    if (!aligned16(p)) return fail(HIPRWKV_EINVAL, "rwkv7_shiftmix_bwd: tensor pointers must be 16-byte aligned");
+  }
+  const int64_t elem = io_dtype == HIPRWKV_F32 ? 4 : 2;
+  if (dprev_batch_stride < C || (dprev_batch_stride * elem) % 16 != 0)
+    return fail(HIPRWKV_EINVAL, "rwkv7_shiftmix_bwd: the batch stride of dprev must be at least C and a multiple of 16 bytes");
+  hipError_t e = launch_rwkv7_shiftmix_bwd(io_dtype == HIPRWKV_F32, B, T, C, n_out, x, prev, prev_batch_stride, new_starts,
+                                           mix, g, dx, dprev, dprev_batch_stride, dmix, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "rwkv7_shiftmix_bwd: %s", hipGetErrorString(e));
+  return HIPRWKV_OK;
 }
 
 int hiprwkv_rwkv7_premix(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t H, int64_t N, const void* k,

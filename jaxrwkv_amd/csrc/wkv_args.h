@@ -110,6 +110,13 @@ hipError_t launch_rwkv7_premix(int io_f32, int64_t rows, int64_t H, const void* 
 hipError_t launch_rwkv7_postmix(int io_f32, int64_t rows, int64_t H, const void* y, const void* r, const void* k,
                                 const void* v, const void* g, const void* ln_w, const void* ln_b, const void* r_k,
                                 float eps, void* out, hipStream_t stream);
+hipError_t launch_rwkv7_shiftmix(int io_f32, int64_t B, int64_t T, int64_t C, int n_out, const void* x, const void* prev,
+                                 int64_t prev_bstride, const uint8_t* ns, const void* const* mix, void* const* out,
+                                 hipStream_t stream);
+hipError_t launch_rwkv7_shiftmix_bwd(int io_f32, int64_t B, int64_t T, int64_t C, int n_out, const void* x,
+                                     const void* prev, int64_t prev_bstride, const uint8_t* ns, const void* const* mix,
+                                     const void* const* g, void* dx, void* dprev, int64_t dprev_bstride, float* dmix,
+                                     hipStream_t stream);
 hipError_t launch_rwkv7_premix_bwd(int io_f32, int64_t rows, int64_t H, const void* k, const void* a, const void* k_k,
                                    const void* k_a, const void* gko, const void* gao, const void* gbo, void* gk,
                                    void* ga, float* gk_k, float* gk_a, hipStream_t stream);

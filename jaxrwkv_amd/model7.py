@@ -116,7 +116,8 @@ class RWKV7:
     """``forward`` / ``default_state`` with the reference's argument names; batched over the leading axis."""
 
     inner = HipRWKV
-    #: use the fused pre/post time-mixing kernels (ops.rwkv7_premix / rwkv7_postmix), with or without autograd
+    #: use the fused kernels beside the recurrence (ops.rwkv7_shiftmix / rwkv7_premix / rwkv7_postmix), with or without
+    #: autograd
     fuse_mix = True
 
     @classmethod
@@ -136,8 +137,10 @@ class RWKV7:
     @classmethod
     def channel_mixing_seq(cls, x, state_row, ffn, last_idx, new_starts):
         """rwkv7.py:190-198"""
-        sx = cls._shift(x, state_row, new_starts)
-        xk = x + sx * ffn["x_k"]
+        if cls.fuse_mix:
+            xk, = ops.rwkv7_shiftmix(x, state_row, new_starts, [ffn["x_k"]])
+        else:
+            xk = x + cls._shift(x, state_row, new_starts) * ffn["x_k"]
         k = torch.square(torch.relu(xk @ ffn["key"]["weight"].T))
         return k @ ffn["value"]["weight"].T, x[torch.arange(x.shape[0], device=x.device), last_idx]
 
@@ -149,8 +152,12 @@ class RWKV7:
         in place and the third result is None."""
         B, T, C = x.shape
         H, N = att["r_k"].shape
-        sx = cls._shift(x, shift_row, new_starts)
-        xr, xw, xk, xv, xa, xg = (x + sx * att[n] for n in ("x_r", "x_w", "x_k", "x_v", "x_a", "x_g"))
+        mix_names = ("x_r", "x_w", "x_k", "x_v", "x_a", "x_g")
+        if cls.fuse_mix:
+            xr, xw, xk, xv, xa, xg = ops.rwkv7_shiftmix(x, shift_row, new_starts, [att[n] for n in mix_names])
+        else:
+            sx = cls._shift(x, shift_row, new_starts)
+            xr, xw, xk, xv, xa, xg = (x + sx * att[n] for n in mix_names)
         r = xr @ att["receptance"]["weight"].T
         w = -F.softplus(-(att["w0"] + torch.tanh(xw @ att["w1"]) @ att["w2"]).float()).to(x.dtype) - 0.5
         k = xk @ att["key"]["weight"].T

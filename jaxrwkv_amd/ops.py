@@ -6,6 +6,8 @@ current stream.  ``compat=True`` (default) reproduces ``AssociativeScanRWKV``; `
 ``BaseRWKV``/``ScanRWKV`` conventions (they differ only in y[t] when new_starts[t+1], and in the returned state
 when new_starts[length]).
 """
+import ctypes
+
 import torch
 
 from . import _lib
@@ -54,7 +56,6 @@ def _flags(compat, force_seq=False, small_t=True, debug=0):
 def handshake_failures():
     """Workgroups of the chunked kernels whose bounded hand-shake wait ran out since the library was loaded (their
     outputs are NaN).  Synchronises the current stream."""
-    import ctypes
     lib = _lib.load()
     n = ctypes.c_uint(0)
     _lib.check(lib.hiprwkv_handshake_failures(_stream(), ctypes.byref(n)), "hiprwkv_handshake_failures")
@@ -396,6 +397,76 @@ class _Postmix(torch.autograd.Function):
                                            _p(gg), _p(gw), _p(gb), _p(grk))
         _lib.check(rc, "hiprwkv_rwkv7_postmix_bwd")
         return gy, gr, gk, gv, gg, gw.to(io), gb.to(io), grk.to(io), None
+
+
+def _ptr_array(tensors):
+    return (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+
+
+def _shift_row(prev, B, C, io):
+    """The token before t = 0 of every sequence as (tensor, batch stride in elements): rows of C contiguous elements,
+    read where they lie when the stride allows it (a row of the packed model state), else from a dense copy."""
+    assert prev.shape == (B, C), (prev.shape, (B, C))
+    if not prev.is_cuda:
+        raise _lib.HipRwkvError("hiprwkv operators need CUDA (ROCm) tensors; there is no CPU path")
+    elem = 4 if io == torch.float32 else 2
+    ok = (prev.dtype == io and (C == 1 or prev.stride(1) == 1) and prev.data_ptr() % 16 == 0
+          and (B == 1 or (prev.stride(0) >= C and (prev.stride(0) * elem) % 16 == 0)))
+    if not ok:
+        prev = prev.to(io).contiguous()
+    return prev, (prev.stride(0) if B > 1 else C)
+
+
+def _shiftmix_fwd(x, prev, prev_stride, ns, mix):
+    lib = _lib.load()
+    io = x.dtype
+    B, T, C = x.shape
+    outs = [torch.empty_like(x) for _ in mix]
+    rc = lib.hiprwkv_rwkv7_shiftmix(_stream(), _DT[io], B, T, C, len(mix), _p(x), _p(prev), prev_stride, _p(ns),
+                                    _ptr_array(mix), _ptr_array(outs))
+    _lib.check(rc, "hiprwkv_rwkv7_shiftmix")
+    return tuple(outs)
+
+
+class _ShiftMix(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, prev, ns, *mix):
+        prev_t, stride = _shift_row(prev, x.shape[0], x.shape[2], x.dtype)
+        ctx.save_for_backward(x, prev_t, *mix)
+        ctx.ns, ctx.stride = ns, stride
+        return _shiftmix_fwd(x, prev_t, stride, ns, mix)
+
+    @staticmethod
+    def backward(ctx, *gs):
+        x, prev, *mix = ctx.saved_tensors
+        lib = _lib.load()
+        io = x.dtype
+        B, T, C = x.shape
+        gs = [_dev(g, io) for g in gs]
+        dx = torch.empty_like(x)
+        dprev = torch.empty((B, C), dtype=io, device=x.device)
+        dmix = torch.empty((len(mix), C), dtype=torch.float32, device=x.device)
+        rc = lib.hiprwkv_rwkv7_shiftmix_bwd(_stream(), _DT[io], B, T, C, len(mix), _p(x), _p(prev), ctx.stride,
+                                            _p(ctx.ns), _ptr_array(mix), _ptr_array(gs), _p(dx), _p(dprev), C, _p(dmix))
+        _lib.check(rc, "hiprwkv_rwkv7_shiftmix_bwd")
+        return (dx, dprev, None) + tuple(dmix[i].to(io) for i in range(len(mix)))
+
+
+def rwkv7_shiftmix(x, prev, new_starts, mix):
+    """Token shift and interpolation of rwkv7.py:226-235 (six ``mix`` vectors, time mixing) and :192-195 (one, channel
+    mixing): x (B,T,C); prev (B,C), the token before t = 0 (a row of the model state; read in place);
+    new_starts (B,T) bool or None; mix a list of (C,) parameters.  Returns the tuple of x + sx*mix_i with
+    sx = (new_starts ? 0 : previous token) - x.  Differentiable in x, prev and the mix vectors."""
+    io = x.dtype
+    B, T, C = x.shape
+    assert len(mix) in (1, 6) and C % 8 == 0, (len(mix), C)
+    x = _dev(x, io)
+    mix2 = [_dev(m.reshape(C), io) for m in mix]
+    _, ns = _length_ns(None, new_starts, B, T, x.device)
+    if torch.is_grad_enabled() and any(t.requires_grad for t in (x, prev, *mix)):
+        return _ShiftMix.apply(x, prev, ns, *mix2)
+    prev_t, stride = _shift_row(prev, B, C, io)
+    return _shiftmix_fwd(x, prev_t, stride, ns, mix2)
 
 
 def rwkv7_premix(k, a, k_k, k_a):

@@ -95,6 +95,17 @@ def test_misaligned_pointers_are_refused_by_every_entry_point():
     assert rc == -1 and b"N=32" in msg()
     rc = lib.hiprwkv_rwkv7_postmix(null, 1, 8, 1, 64, ok, bad, ok, ok, ok, ok, ok, ok, 1e-5, ok)
     assert rc == -1 and b"aligned" in msg()
+    # token shift + interpolation: pointer arrays in host memory, C a multiple of 8, one or six outputs
+    arr = lambda *ps: (ctypes.c_void_p * len(ps))(*[p.value for p in ps])
+    six_ok, six_bad = arr(*([ok] * 6)), arr(ok, ok, ok, bad, ok, ok)
+    assert lib.hiprwkv_rwkv7_shiftmix(null, 1, 2, 8, 64, 6, ok, ok, 64, null, six_ok, six_bad) == -1 and b"aligned" in msg()
+    assert lib.hiprwkv_rwkv7_shiftmix(null, 1, 2, 8, 60, 6, ok, ok, 64, null, six_ok, six_ok) == -1 and b"multiple of 8" in msg()
+    assert lib.hiprwkv_rwkv7_shiftmix(null, 1, 2, 8, 64, 3, ok, ok, 64, null, six_ok, six_ok) == -1 and b"n_out" in msg()
+    assert lib.hiprwkv_rwkv7_shiftmix(null, 1, 2, 8, 64, 1, ok, ok, 60, null, six_ok, six_ok) == -1 and b"stride" in msg()
+    assert lib.hiprwkv_rwkv7_shiftmix(null, 1, 2, 8, 64, 1, ok, null, 64, null, six_ok, six_ok) == -1 and b"null" in msg()
+    assert lib.hiprwkv_rwkv7_shiftmix_bwd(null, 1, 2, 8, 64, 6, ok, ok, 64, null, six_ok, six_bad, ok, ok, 64, ok) == -1
+    assert lib.hiprwkv_rwkv7_shiftmix_bwd(null, 1, 2, 8, 64, 6, ok, ok, 64, null, six_ok, six_ok, ok, ok, 64, null) == -1 and b"null" in msg()
+    assert lib.hiprwkv_rwkv7_shiftmix_bwd(null, 1, 2, 8, 64, 6, ok, ok, 64, null, six_ok, six_ok, ok, ok, 12, ok) == -1 and b"dprev" in msg()
 
 
 def test_cpu_tensors_are_refused_loudly():

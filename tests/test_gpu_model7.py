@@ -210,6 +210,64 @@ def test_fused_time_mixing_stages_backward_against_torch_autograd(dtype, rows):
             torch.testing.assert_close(gg, gw, rtol=2.0 ** -6, atol=2e-2 * scale, msg=lambda m: f"{name}: {m}")
 
 
+def _shift_reference(x, prev, ns, mix):
+    """rwkv7.py:226-235 / :192-195 in plain torch fp32: concatenate, zero at new_starts, subtract, interpolate."""
+    xf = x.float()            # one conversion: the cotangent of x is then rounded to x's dtype once, as in the kernel
+    sx = torch.cat([prev.float()[:, None], xf[:, :-1]], dim=1)
+    sx = torch.where(ns[:, :, None], torch.zeros_like(sx), sx) - xf
+    return tuple(xf + sx * m.float() for m in mix)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n_out", [1, 6])
+@pytest.mark.parametrize("shape", [(3, 37, 128), (1, 1, 64), (2, 300, 2048 + 64)])
+def test_token_shift_interpolation_forward_and_backward_against_torch(dtype, n_out, shape):
+    """ops.rwkv7_shiftmix, values and all cotangents (x, the state row, the interpolation vectors), against torch
+    autograd of the plain formula.  The state row is read where it lies inside a packed model state; new_starts hits
+    t = 0, the last token and ordinary tokens."""
+    from jaxrwkv_amd import ops
+    B, T, C = shape
+    g = torch.Generator("cuda").manual_seed(21 + n_out)
+    n = lambda *s: torch.randn(s, device="cuda", generator=g).to(dtype)
+    x = n(B, T, C)
+    state = n(B, 3, 5, C)                       # a model state (B, L, rows, C); the shift row of layer 1 is row 1
+    mix = [torch.rand(C, device="cuda", generator=g).to(dtype) for _ in range(n_out)]
+    ns = torch.rand((B, T), device="cuda", generator=g) < 0.2
+    ns[0, 0] = True
+    ns[-1, -1] = True
+    cot = [n(B, T, C) for _ in range(n_out)]
+    leaf = lambda t: t.detach().clone().requires_grad_()
+    loss = lambda outs: sum((o.float() * c.float()).sum() for o, c in zip(outs, cot))
+
+    fx, fstate, fmix = leaf(x), leaf(state), [leaf(m) for m in mix]
+    outs = ops.rwkv7_shiftmix(fx, fstate[:, 1, 1], ns, fmix)
+    loss(outs).backward()
+    rx, rstate, rmix = leaf(x), leaf(state), [leaf(m) for m in mix]
+    refs = _shift_reference(rx, rstate[:, 1, 1], ns, rmix)
+    loss(refs).backward()
+
+    tol = dict(rtol=1e-6, atol=1e-6) if dtype == torch.float32 else dict(rtol=2.0 ** -8, atol=1e-6)
+    for o, r in zip(outs, refs):
+        assert o.dtype == dtype
+        torch.testing.assert_close(o.float(), r, **tol)
+    with torch.no_grad():                        # the path without autograd gives the same values
+        plain = ops.rwkv7_shiftmix(x, state[:, 1, 1], ns, mix)
+    assert all(torch.equal(a, b) for a, b in zip(plain, outs))
+    pairs = [("x", fx, rx), ("state", fstate, rstate)] + [(f"mix{i}", a, b) for i, (a, b) in enumerate(zip(fmix, rmix))]
+    for name, got, want in pairs:
+        assert got.grad is not None and got.grad.dtype == dtype and got.grad.shape == want.grad.shape, name
+        gw, gg = want.grad.float(), got.grad.float()
+        scale = float(gw.pow(2).mean().sqrt()) + 1e-30
+        if dtype == torch.float32:
+            torch.testing.assert_close(gg, gw, rtol=1e-4, atol=1e-5 * scale, msg=lambda m: f"{name}: {m}")
+        else:
+            torch.testing.assert_close(gg, gw, rtol=2.0 ** -7, atol=1e-2 * scale, msg=lambda m: f"{name}: {m}")
+    # nothing but the shift row of layer 1 receives a cotangent
+    mask = torch.ones_like(fstate.grad, dtype=torch.bool)
+    mask[:, 1, 1] = False
+    assert bool((fstate.grad[mask] == 0).all())
+
+
 def test_model_gradients_with_and_without_fused_stages_agree():
     """Training-style use: d(loss)/d(params) through the whole model with the fused stages' backward kernels against
     the same model on plain torch ops around the same WKV kernels."""
