@@ -209,6 +209,24 @@ int hiprwkv_rwkv7_shiftmix_bwd(hiprwkv_stream stream, int io_dtype, int64_t B, i
                                const void* const* mix, const void* const* g, void* dx, void* dprev,
                                int64_t dprev_batch_stride, float* dmix);
 
+/* ---- RWKV-7 decay, value mix and gate between the projections and the op -------------------
+ * Element-wise steps of time_mixing_seq that the reference computes in jnp (rwkv7.py:237, :241-242, :244); no
+ * counterpart among its ffi targets.  Token tensors (rows, C) io_dtype, parameters w0, v0, a0 (C,) io_dtype, C a
+ * multiple of 8; the parameter cotangents dw0, dv0, da0 are (C,) fp32 sums over the rows (zeroed by the call).
+ *     decay:  w  = -softplus(-(w0 + x)) - 0.5          x = tanh(xw w1) w2
+ *     vmix :  v' = v + (v_first - v) sigmoid(v0 + x)   x = (xv v1) v2      (layers after the first)
+ *     agate:  a  = sigmoid(a0 + x)                     x = (xa a1) a2 */
+int hiprwkv_rwkv7_decay(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t C, const void* x, const void* w0, void* w);
+int hiprwkv_rwkv7_decay_bwd(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t C, const void* x, const void* w0,
+                            const void* g, void* dx, float* dw0);
+int hiprwkv_rwkv7_agate(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t C, const void* x, const void* a0, void* a);
+int hiprwkv_rwkv7_agate_bwd(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t C, const void* x, const void* a0,
+                            const void* g, void* dx, float* da0);
+int hiprwkv_rwkv7_vmix(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t C, const void* v, const void* v_first,
+                       const void* x, const void* v0, void* out);
+int hiprwkv_rwkv7_vmix_bwd(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t C, const void* v, const void* v_first,
+                           const void* x, const void* v0, const void* g, void* dv, void* dv_first, void* dx, float* dv0);
+
 /* ---- RWKV-7 time-mixing stages around the op ------------------------------------------
  * The element-wise work the reference does in jnp on either side of inner_loop (rwkv7.py:248-252, 257 and :263-265),
  * fused into one pass each; it has no counterpart among the reference's ffi targets.  `rows` = number of tokens

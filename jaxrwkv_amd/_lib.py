@@ -43,6 +43,12 @@ SIGNATURES = {
     "hiprwkv_wkv4_bwd_noalloc": (_int, [_vp, _int, _i64, _i64, _i64] + [_vp] * 6 + [_vp, _vp] + [_vp] + [_vp] * 5 + [_u32]),
     "hiprwkv_rwkv7_shiftmix": (_int, [_vp, _int, _i64, _i64, _i64, _int, _vp, _vp, _i64, _vp, _vp, _vp]),
     "hiprwkv_rwkv7_shiftmix_bwd": (_int, [_vp, _int, _i64, _i64, _i64, _int, _vp, _vp, _i64, _vp, _vp, _vp, _vp, _vp, _i64, _vp]),
+    "hiprwkv_rwkv7_decay": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _vp]),
+    "hiprwkv_rwkv7_decay_bwd": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _vp, _vp, _vp]),
+    "hiprwkv_rwkv7_agate": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _vp]),
+    "hiprwkv_rwkv7_agate_bwd": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _vp, _vp, _vp]),
+    "hiprwkv_rwkv7_vmix": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _vp, _vp, _vp]),
+    "hiprwkv_rwkv7_vmix_bwd": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "hiprwkv_rwkv7_premix": (_int, [_vp, _int, _i64, _i64, _i64] + [_vp] * 7),
     "hiprwkv_rwkv7_postmix": (_int, [_vp, _int, _i64, _i64, _i64] + [_vp] * 8 + [ctypes.c_float, _vp]),
     "hiprwkv_rwkv7_premix_bwd": (_int, [_vp, _int, _i64, _i64, _i64] + [_vp] * 11),

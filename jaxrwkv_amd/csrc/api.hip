@@ -5,6 +5,7 @@
 #include <stdio.h>
 #include <string.h>
 
+#include <initializer_list>
 #include <mutex>
 
 #include "wkv_args.h"
@@ -93,7 +94,7 @@ unsigned* status_word() {
 extern "C" {
 
 const char* hiprwkv_last_error(void) { return g_err; }
-int hiprwkv_version(void) { return 104; }
+int hiprwkv_version(void) { return 105; }
 
 int hiprwkv_handshake_failures(hiprwkv_stream stream, unsigned* count) {
   if (count == nullptr) return fail(HIPRWKV_EINVAL, "handshake_failures: null count pointer");
@@ -449,6 +450,52 @@ int hiprwkv_rwkv7_shiftmix_bwd(hiprwkv_stream stream, int io_dtype, int64_t B, i
                                            mix, g, dx, dprev, dprev_batch_stride, dmix, static_cast<hipStream_t>(stream));
   if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "rwkv7_shiftmix_bwd: %s", hipGetErrorString(e));
   return HIPRWKV_OK;
+}
+
+namespace {
+int check_gate(const char* op, int io_dtype, int64_t rows, int64_t C, std::initializer_list<const void*> ptrs) {
+  if (!dtype_ok(io_dtype)) return fail(HIPRWKV_EINVAL, "%s: dtype must be HIPRWKV_F32 or HIPRWKV_BF16", op);
+  if (rows <= 0 || C <= 0 || C % 8 != 0) return fail(HIPRWKV_EINVAL, "%s: rows must be positive and C a positive multiple of 8", op);
+  if (rows * (C / 8) > 0x7fffffffLL * 256) return fail(HIPRWKV_EINVAL, "%s: too many elements for one launch", op);
+  for (const void* p : ptrs) {
+    if (p == nullptr) return fail(HIPRWKV_EINVAL, "%s: null tensor pointer", op);
+    if (!aligned16(p)) return fail(HIPRWKV_EINVAL, "%s: tensor pointers must be 16-byte aligned", op);
+  }
+  return HIPRWKV_OK;
+}
+int gate_done(const char* op, hipError_t e) {
+  if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "%s: %s", op, hipGetErrorString(e));
+  return HIPRWKV_OK;
+}
+}  // namespace
+
+int hiprwkv_rwkv7_decay(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t C, const void* x, const void* w0, void* w) {
+  if (int rc = check_gate("rwkv7_decay", io_dtype, rows, C, {x, w0, w})) return rc;
+  return gate_done("rwkv7_decay", launch_rwkv7_decay(io_dtype == HIPRWKV_F32, 0, rows, C, x, w0, w, static_cast<hipStream_t>(stream)));
+}
+int hiprwkv_rwkv7_decay_bwd(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t C, const void* x, const void* w0,
+                            const void* g, void* dx, float* dw0) {
+  if (int rc = check_gate("rwkv7_decay_bwd", io_dtype, rows, C, {x, w0, g, dx, dw0})) return rc;
+  return gate_done("rwkv7_decay_bwd", launch_rwkv7_decay_bwd(io_dtype == HIPRWKV_F32, 0, rows, C, x, w0, g, dx, dw0, static_cast<hipStream_t>(stream)));
+}
+int hiprwkv_rwkv7_agate(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t C, const void* x, const void* a0, void* a) {
+  if (int rc = check_gate("rwkv7_agate", io_dtype, rows, C, {x, a0, a})) return rc;
+  return gate_done("rwkv7_agate", launch_rwkv7_decay(io_dtype == HIPRWKV_F32, 1, rows, C, x, a0, a, static_cast<hipStream_t>(stream)));
+}
+int hiprwkv_rwkv7_agate_bwd(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t C, const void* x, const void* a0,
+                            const void* g, void* dx, float* da0) {
+  if (int rc = check_gate("rwkv7_agate_bwd", io_dtype, rows, C, {x, a0, g, dx, da0})) return rc;
+  return gate_done("rwkv7_agate_bwd", launch_rwkv7_decay_bwd(io_dtype == HIPRWKV_F32, 1, rows, C, x, a0, g, dx, da0, static_cast<hipStream_t>(stream)));
+}
+int hiprwkv_rwkv7_vmix(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t C, const void* v, const void* v_first,
+                       const void* x, const void* v0, void* out) {
+  if (int rc = check_gate("rwkv7_vmix", io_dtype, rows, C, {v, v_first, x, v0, out})) return rc;
+  return gate_done("rwkv7_vmix", launch_rwkv7_vmix(io_dtype == HIPRWKV_F32, rows, C, v, v_first, x, v0, out, static_cast<hipStream_t>(stream)));
+}
+int hiprwkv_rwkv7_vmix_bwd(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t C, const void* v, const void* v_first,
+                           const void* x, const void* v0, const void* g, void* dv, void* dv_first, void* dx, float* dv0) {
+  if (int rc = check_gate("rwkv7_vmix_bwd", io_dtype, rows, C, {v, v_first, x, v0, g, dv, dv_first, dx, dv0})) return rc;
+  return gate_done("rwkv7_vmix_bwd", launch_rwkv7_vmix_bwd(io_dtype == HIPRWKV_F32, rows, C, v, v_first, x, v0, g, dv, dv_first, dx, dv0, static_cast<hipStream_t>(stream)));
 }
 
 int hiprwkv_rwkv7_premix(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t H, int64_t N, const void* k,

@@ -110,6 +110,15 @@ hipError_t launch_rwkv7_premix(int io_f32, int64_t rows, int64_t H, const void* 
 hipError_t launch_rwkv7_postmix(int io_f32, int64_t rows, int64_t H, const void* y, const void* r, const void* k,
                                 const void* v, const void* g, const void* ln_w, const void* ln_b, const void* r_k,
                                 float eps, void* out, hipStream_t stream);
+hipError_t launch_rwkv7_decay(int io_f32, int sigmoid, int64_t rows, int64_t C, const void* x, const void* w0, void* w,
+                              hipStream_t stream);
+hipError_t launch_rwkv7_decay_bwd(int io_f32, int sigmoid, int64_t rows, int64_t C, const void* x, const void* w0,
+                                  const void* g, void* dx, float* dw0, hipStream_t stream);
+hipError_t launch_rwkv7_vmix(int io_f32, int64_t rows, int64_t C, const void* v, const void* v_first, const void* x,
+                             const void* v0, void* out, hipStream_t stream);
+hipError_t launch_rwkv7_vmix_bwd(int io_f32, int64_t rows, int64_t C, const void* v, const void* v_first, const void* x,
+                                 const void* v0, const void* g, void* dv, void* dv_first, void* dx, float* dv0,
+                                 hipStream_t stream);
 hipError_t launch_rwkv7_shiftmix(int io_f32, int64_t B, int64_t T, int64_t C, int n_out, const void* x, const void* prev,
                                  int64_t prev_bstride, const uint8_t* ns, const void* const* mix, void* const* out,
                                  hipStream_t stream);

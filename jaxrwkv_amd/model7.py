@@ -116,8 +116,8 @@ class RWKV7:
     """``forward`` / ``default_state`` with the reference's argument names; batched over the leading axis."""
 
     inner = HipRWKV
-    #: use the fused kernels beside the recurrence (ops.rwkv7_shiftmix / rwkv7_premix / rwkv7_postmix), with or without
-    #: autograd
+    #: use the fused kernels beside the recurrence (ops.rwkv7_shiftmix, rwkv7_decay, rwkv7_vmix, rwkv7_agate,
+    #: rwkv7_premix, rwkv7_postmix), with or without autograd
     fuse_mix = True
 
     @classmethod
@@ -159,14 +159,23 @@ class RWKV7:
             sx = cls._shift(x, shift_row, new_starts)
             xr, xw, xk, xv, xa, xg = (x + sx * att[n] for n in mix_names)
         r = xr @ att["receptance"]["weight"].T
-        w = -F.softplus(-(att["w0"] + torch.tanh(xw @ att["w1"]) @ att["w2"]).float()).to(x.dtype) - 0.5
+        w_lora = torch.tanh(xw @ att["w1"]) @ att["w2"]
+        if cls.fuse_mix:
+            w = ops.rwkv7_decay(w_lora, att["w0"])
+        else:
+            w = -F.softplus(-(att["w0"] + w_lora).float()).to(x.dtype) - 0.5
         k = xk @ att["key"]["weight"].T
         v = xv @ att["value"]["weight"].T
         if layer_id == 0:
             v_first = v
         else:
-            v = v + (v_first - v) * torch.sigmoid(att["v0"] + (xv @ att["v1"]) @ att["v2"])
-        a = torch.sigmoid(att["a0"] + (xa @ att["a1"]) @ att["a2"])
+            v_lora = (xv @ att["v1"]) @ att["v2"]
+            if cls.fuse_mix:
+                v = ops.rwkv7_vmix(v, v_first, v_lora, att["v0"])
+            else:
+                v = v + (v_first - v) * torch.sigmoid(att["v0"] + v_lora)
+        a_lora = (xa @ att["a1"]) @ att["a2"]
+        a = ops.rwkv7_agate(a_lora, att["a0"]) if cls.fuse_mix else torch.sigmoid(att["a0"] + a_lora)
         g = torch.sigmoid(xg @ att["g1"]) @ att["g2"]
         new_shift = x[torch.arange(B, device=x.device), last_idx]
         fused = cls.fuse_mix

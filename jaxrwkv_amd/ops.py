@@ -469,6 +469,103 @@ def rwkv7_shiftmix(x, prev, new_starts, mix):
     return _shiftmix_fwd(x, prev_t, stride, ns, mix2)
 
 
+def _gate_fwd(x, p, kind):
+    lib = _lib.load()
+    io = x.dtype
+    C = x.shape[-1]
+    out = torch.empty_like(x)
+    fn = (lib.hiprwkv_rwkv7_decay, lib.hiprwkv_rwkv7_agate)[kind]
+    _lib.check(fn(_stream(), _DT[io], x.numel() // C, C, _p(x), _p(p), _p(out)), "hiprwkv_rwkv7_" + ("decay", "agate")[kind])
+    return out
+
+
+class _Gate(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x, p, kind):
+        ctx.save_for_backward(x, p)
+        ctx.kind = kind
+        return _gate_fwd(x, p, kind)
+
+    @staticmethod
+    def backward(ctx, g):
+        x, p = ctx.saved_tensors
+        lib = _lib.load()
+        io = x.dtype
+        C = x.shape[-1]
+        g = _dev(g, io)
+        dx = torch.empty_like(x)
+        dp = torch.empty(C, dtype=torch.float32, device=x.device)
+        fn = (lib.hiprwkv_rwkv7_decay_bwd, lib.hiprwkv_rwkv7_agate_bwd)[ctx.kind]
+        _lib.check(fn(_stream(), _DT[io], x.numel() // C, C, _p(x), _p(p), _p(g), _p(dx), _p(dp)),
+                   "hiprwkv_rwkv7_" + ("decay", "agate")[ctx.kind] + "_bwd")
+        return dx, dp.to(io), None
+
+
+def _gate(x, p, kind):
+    io = x.dtype
+    C = x.shape[-1]
+    assert C % 8 == 0, C
+    x, p2 = _dev(x, io), _dev(p.reshape(C), io)
+    if torch.is_grad_enabled() and (x.requires_grad or p.requires_grad):
+        return _Gate.apply(x, p2, kind)
+    return _gate_fwd(x, p2, kind)
+
+
+def rwkv7_decay(x, w0):
+    """The decay argument of the WKV op, rwkv7.py:237: ``-softplus(-(w0 + x)) - 0.5`` for x (..., C) (the low-rank
+    term ``tanh(xw w1) w2``) and the parameter w0 (C,).  Differentiable in both."""
+    return _gate(x, w0, 0)
+
+
+def rwkv7_agate(x, a0):
+    """The in-context learning rate, rwkv7.py:244: ``sigmoid(a0 + x)`` for x (..., C) and a0 (C,).  Differentiable."""
+    return _gate(x, a0, 1)
+
+
+def _vmix_fwd(v, vf, x, v0):
+    lib = _lib.load()
+    io = v.dtype
+    C = v.shape[-1]
+    out = torch.empty_like(v)
+    rc = lib.hiprwkv_rwkv7_vmix(_stream(), _DT[io], v.numel() // C, C, _p(v), _p(vf), _p(x), _p(v0), _p(out))
+    _lib.check(rc, "hiprwkv_rwkv7_vmix")
+    return out
+
+
+class _VMix(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, v, vf, x, v0):
+        ctx.save_for_backward(v, vf, x, v0)
+        return _vmix_fwd(v, vf, x, v0)
+
+    @staticmethod
+    def backward(ctx, g):
+        v, vf, x, v0 = ctx.saved_tensors
+        lib = _lib.load()
+        io = v.dtype
+        C = v.shape[-1]
+        g = _dev(g, io)
+        dv, dvf, dx = (torch.empty_like(v) for _ in range(3))
+        dv0 = torch.empty(C, dtype=torch.float32, device=v.device)
+        rc = lib.hiprwkv_rwkv7_vmix_bwd(_stream(), _DT[io], v.numel() // C, C, _p(v), _p(vf), _p(x), _p(v0), _p(g),
+                                        _p(dv), _p(dvf), _p(dx), _p(dv0))
+        _lib.check(rc, "hiprwkv_rwkv7_vmix_bwd")
+        return dv, dvf, dx, dv0.to(io)
+
+
+def rwkv7_vmix(v, v_first, x, v0):
+    """The value residual of the layers after the first, rwkv7.py:241-242: ``v + (v_first - v) sigmoid(v0 + x)`` for
+    v, v_first, x (..., C) (x the low-rank term ``(xv v1) v2``) and the parameter v0 (C,).  Differentiable in all four."""
+    io = v.dtype
+    C = v.shape[-1]
+    assert C % 8 == 0, C
+    v, vf, x = (_dev(t, io) for t in (v, v_first, x))
+    v02 = _dev(v0.reshape(C), io)
+    if torch.is_grad_enabled() and any(t.requires_grad for t in (v, v_first, x, v0)):
+        return _VMix.apply(v, vf, x, v02)
+    return _vmix_fwd(v, vf, x, v02)
+
+
 def rwkv7_premix(k, a, k_k, k_a):
     """k, a (..., H, N); k_k, k_a (H, N) or (H*N,).  Returns (k', a_i, b_i) of rwkv7.py:248-252, 257:
     kk = normalize_head(k k_k), k' = k (1 + (a - 1) k_a), a_i = -kk, b_i = kk a.  Differentiable in all four inputs

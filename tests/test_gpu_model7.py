@@ -268,6 +268,47 @@ def test_token_shift_interpolation_forward_and_backward_against_torch(dtype, n_o
     assert bool((fstate.grad[mask] == 0).all())
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(3, 37, 128), (1, 1, 64), (2, 300, 2048 + 64)])
+def test_decay_value_mix_and_gate_forward_and_backward_against_torch(dtype, shape):
+    """ops.rwkv7_decay / rwkv7_vmix / rwkv7_agate (rwkv7.py:237, :241-242, :244), values and all cotangents, against
+    torch autograd of the plain formulas in fp32 on the same (dtype-rounded) inputs."""
+    from jaxrwkv_amd import ops
+    B, T, C = shape
+    g = torch.Generator("cuda").manual_seed(31)
+    n = lambda *s, scale=1.0: (scale * torch.randn(s, device="cuda", generator=g)).to(dtype)
+    leaf = lambda t: t.detach().clone().requires_grad_()
+    x, v, vf, cot = n(B, T, C, scale=3.0), n(B, T, C), n(B, T, C), n(B, T, C)
+    p = n(C, scale=2.0)
+    cases = {
+        "decay": (lambda x_, p_: ops.rwkv7_decay(x_, p_),
+                  lambda x_, p_: -torch.nn.functional.softplus(-(p_.float() + x_.float())) - 0.5, (x, p)),
+        "agate": (lambda x_, p_: ops.rwkv7_agate(x_, p_), lambda x_, p_: torch.sigmoid(p_.float() + x_.float()), (x, p)),
+        # every input converted once: its cotangent is then rounded to the input's dtype once, as in the kernel
+        "vmix": (lambda v_, f_, x_, p_: ops.rwkv7_vmix(v_, f_, x_, p_),
+                 lambda v_, f_, x_, p_: (lambda v32: v32 + (f_.float() - v32) * torch.sigmoid(p_.float() + x_.float()))(v_.float()),
+                 (v, vf, x, p)),
+    }
+    for name, (fused, plain, inputs) in cases.items():
+        fi, ri = [leaf(t) for t in inputs], [leaf(t) for t in inputs]
+        out, ref = fused(*fi), plain(*ri)
+        assert out.dtype == dtype and out.shape == ref.shape, name
+        tol = dict(rtol=1e-5, atol=1e-6) if dtype == torch.float32 else dict(rtol=2.0 ** -8, atol=1e-6)
+        torch.testing.assert_close(out.float(), ref, msg=lambda m: f"{name}: {m}", **tol)
+        with torch.no_grad():
+            assert torch.equal(fused(*inputs), out), name
+        (out.float() * cot.float()).sum().backward()
+        (ref * cot.float()).sum().backward()
+        for i, (a, b) in enumerate(zip(fi, ri)):
+            assert a.grad is not None and a.grad.dtype == dtype and a.grad.shape == b.grad.shape, (name, i)
+            gw, gg = b.grad.float(), a.grad.float()
+            scale = float(gw.pow(2).mean().sqrt()) + 1e-30
+            if dtype == torch.float32:
+                torch.testing.assert_close(gg, gw, rtol=1e-4, atol=1e-5 * scale, msg=lambda m: f"{name} input {i}: {m}")
+            else:
+                torch.testing.assert_close(gg, gw, rtol=2.0 ** -7, atol=1e-2 * scale, msg=lambda m: f"{name} input {i}: {m}")
+
+
 def test_model_gradients_with_and_without_fused_stages_agree():
     """Training-style use: d(loss)/d(params) through the whole model with the fused stages' backward kernels against
     the same model on plain torch ops around the same WKV kernels."""
