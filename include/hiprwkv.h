@@ -222,6 +222,9 @@ int hiprwkv_rwkv7_decay_bwd(hiprwkv_stream stream, int io_dtype, int64_t rows, i
 int hiprwkv_rwkv7_agate(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t C, const void* x, const void* a0, void* a);
 int hiprwkv_rwkv7_agate_bwd(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t C, const void* x, const void* a0,
                             const void* g, void* dx, float* da0);
+/* Channel mixing's activation, rwkv7.py:196: out = relu(x)^2 over n elements (n a multiple of 8); dx = 2 g relu(x). */
+int hiprwkv_rwkv7_relusq(hiprwkv_stream stream, int io_dtype, int64_t n, const void* x, void* out);
+int hiprwkv_rwkv7_relusq_bwd(hiprwkv_stream stream, int io_dtype, int64_t n, const void* x, const void* g, void* dx);
 int hiprwkv_rwkv7_vmix(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t C, const void* v, const void* v_first,
                        const void* x, const void* v0, void* out);
 int hiprwkv_rwkv7_vmix_bwd(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t C, const void* v, const void* v_first,

@@ -47,6 +47,8 @@ SIGNATURES = {
     "hiprwkv_rwkv7_decay_bwd": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _vp, _vp, _vp]),
     "hiprwkv_rwkv7_agate": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _vp]),
     "hiprwkv_rwkv7_agate_bwd": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _vp, _vp, _vp]),
+    "hiprwkv_rwkv7_relusq": (_int, [_vp, _int, _i64, _vp, _vp]),
+    "hiprwkv_rwkv7_relusq_bwd": (_int, [_vp, _int, _i64, _vp, _vp, _vp]),
     "hiprwkv_rwkv7_vmix": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _vp, _vp, _vp]),
     "hiprwkv_rwkv7_vmix_bwd": (_int, [_vp, _int, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "hiprwkv_rwkv7_premix": (_int, [_vp, _int, _i64, _i64, _i64] + [_vp] * 7),

@@ -94,7 +94,7 @@ unsigned* status_word() {
 extern "C" {
 
 const char* hiprwkv_last_error(void) { return g_err; }
-int hiprwkv_version(void) { return 105; }
+int hiprwkv_version(void) { return 106; }
 
 int hiprwkv_handshake_failures(hiprwkv_stream stream, unsigned* count) {
   if (count == nullptr) return fail(HIPRWKV_EINVAL, "handshake_failures: null count pointer");
@@ -486,6 +486,14 @@ int hiprwkv_rwkv7_agate_bwd(hiprwkv_stream stream, int io_dtype, int64_t rows, i
                             const void* g, void* dx, float* da0) {
   if (int rc = check_gate("rwkv7_agate_bwd", io_dtype, rows, C, {x, a0, g, dx, da0})) return rc;
   return gate_done("rwkv7_agate_bwd", launch_rwkv7_decay_bwd(io_dtype == HIPRWKV_F32, 1, rows, C, x, a0, g, dx, da0, static_cast<hipStream_t>(stream)));
+}
+int hiprwkv_rwkv7_relusq(hiprwkv_stream stream, int io_dtype, int64_t n, const void* x, void* out) {
+  if (int rc = check_gate("rwkv7_relusq", io_dtype, 1, n, {x, out})) return rc;
+  return gate_done("rwkv7_relusq", launch_rwkv7_relusq(io_dtype == HIPRWKV_F32, n, x, nullptr, out, static_cast<hipStream_t>(stream)));
+}
+int hiprwkv_rwkv7_relusq_bwd(hiprwkv_stream stream, int io_dtype, int64_t n, const void* x, const void* g, void* dx) {
+  if (int rc = check_gate("rwkv7_relusq_bwd", io_dtype, 1, n, {x, g, dx})) return rc;
+  return gate_done("rwkv7_relusq_bwd", launch_rwkv7_relusq(io_dtype == HIPRWKV_F32, n, x, g, dx, static_cast<hipStream_t>(stream)));
 }
 int hiprwkv_rwkv7_vmix(hiprwkv_stream stream, int io_dtype, int64_t rows, int64_t C, const void* v, const void* v_first,
                        const void* x, const void* v0, void* out) {

@@ -3,6 +3,7 @@
 //     decay:  w  = -softplus(-(w0 + x)) - 0.5                 x = tanh(xw w1) w2, the low-rank decay term
 //     vmix :  v' = v + (v_first - v) sigmoid(v0 + x)          x = (xv v1) v2, layers after the first
 //     agate:  a  = sigmoid(a0 + x)                            x = (xa a1) a2
+//     relusq: k  = relu(x)^2                                  channel mixing, rwkv7.py:196 (x = xk W_key)
 // w0, v0, a0 are (C,) parameters, everything else (rows, C).  As separate tensor operations these are five to seven passes
 // over a (T, C) tensor each.  A thread owns eight consecutive channels; fp32 arithmetic, one rounding per output.
 //
@@ -10,6 +11,7 @@
 //     decay:  dx = g sigmoid(-(w0 + x)) ;                      dw0 = sum over rows of dx
 //     vmix :  s = sigmoid(v0 + x) ;  dv = g (1 - s) ;  dv_first = g s ;  dx = g (v_first - v) s (1 - s) ;  dv0 = sum of dx
 //     agate:  dx = g a (1 - a) ;                               da0 = sum of dx
+//     relusq: dx = 2 g relu(x)
 // A workgroup walks a run of rows with the partial sums of the parameter cotangent in registers (a thread's own
 // channels) and ends with one fp32 atomic per channel; the launcher zeroes the result first with a fill kernel.
 #include "common.h"
@@ -54,6 +56,23 @@ __global__ __launch_bounds__(GATE_THREADS) void rwkv7_vmix_kernel(int64_t rows, 
 #pragma unroll
   for (int c = 0; c < 8; ++c) o[c] = fmaf(fv[c] - vv[c], sigmoidf(p[c] + xv[c]), vv[c]);
   st8(out + el, o);
+}
+
+// relu(x)^2 (BWD: 2 g relu(x)) over n8 groups of eight consecutive elements
+template <typename T, bool BWD>
+__global__ __launch_bounds__(GATE_THREADS) void rwkv7_relusq_kernel(int64_t n8, const T* __restrict__ x,
+                                                                     const T* __restrict__ g, T* __restrict__ out) {
+  const int64_t idx = (int64_t)blockIdx.x * GATE_THREADS + threadIdx.x;
+  if (idx >= n8) return;
+  float xv[8], gv[8], o[8];
+  ld8(x + idx * 8, xv);
+  if (BWD) ld8(g + idx * 8, gv);
+#pragma unroll
+  for (int c = 0; c < 8; ++c) {
+    const float r = fmaxf(xv[c], 0.f);
+    o[c] = BWD ? 2.f * gv[c] * r : r * r;
+  }
+  st8(out + idx * 8, o);
 }
 
 // Workgroup (blockIdx.x = channel block, blockIdx.y = run of `run` consecutive rows)
@@ -158,6 +177,18 @@ hipError_t launch_rwkv7_decay_bwd(int io_f32, int sigmoid, int64_t rows, int64_t
                      (const TY*)w0, (const TY*)g, (TY*)dx, dw0)
   if (io_f32) { if (sigmoid) HIPRWKV_GATE_LAUNCH(float, true); else HIPRWKV_GATE_LAUNCH(float, false); }
   else { if (sigmoid) HIPRWKV_GATE_LAUNCH(bf16_t, true); else HIPRWKV_GATE_LAUNCH(bf16_t, false); }
+#undef HIPRWKV_GATE_LAUNCH
+  return hipGetLastError();
+}
+
+// g == nullptr: forward (out = relu(x)^2); else backward (out = 2 g relu(x))
+hipError_t launch_rwkv7_relusq(int io_f32, int64_t n, const void* x, const void* g, void* out, hipStream_t stream) {
+  const int64_t n8 = n / 8;
+  const dim3 grid((unsigned)((n8 + GATE_THREADS - 1) / GATE_THREADS)), block(GATE_THREADS);
+#define HIPRWKV_GATE_LAUNCH(TY, BW) \
+  hipLaunchKernelGGL((rwkv7_relusq_kernel<TY, BW>), grid, block, 0, stream, n8, (const TY*)x, (const TY*)g, (TY*)out)
+  if (io_f32) { if (g) HIPRWKV_GATE_LAUNCH(float, true); else HIPRWKV_GATE_LAUNCH(float, false); }
+  else { if (g) HIPRWKV_GATE_LAUNCH(bf16_t, true); else HIPRWKV_GATE_LAUNCH(bf16_t, false); }
 #undef HIPRWKV_GATE_LAUNCH
   return hipGetLastError();
 }

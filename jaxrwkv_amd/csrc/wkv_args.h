@@ -114,6 +114,7 @@ hipError_t launch_rwkv7_decay(int io_f32, int sigmoid, int64_t rows, int64_t C, 
                               hipStream_t stream);
 hipError_t launch_rwkv7_decay_bwd(int io_f32, int sigmoid, int64_t rows, int64_t C, const void* x, const void* w0,
                                   const void* g, void* dx, float* dw0, hipStream_t stream);
+hipError_t launch_rwkv7_relusq(int io_f32, int64_t n, const void* x, const void* g, void* out, hipStream_t stream);
 hipError_t launch_rwkv7_vmix(int io_f32, int64_t rows, int64_t C, const void* v, const void* v_first, const void* x,
                              const void* v0, void* out, hipStream_t stream);
 hipError_t launch_rwkv7_vmix_bwd(int io_f32, int64_t rows, int64_t C, const void* v, const void* v_first, const void* x,

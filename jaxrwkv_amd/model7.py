@@ -141,7 +141,8 @@ class RWKV7:
             xk, = ops.rwkv7_shiftmix(x, state_row, new_starts, [ffn["x_k"]])
         else:
             xk = x + cls._shift(x, state_row, new_starts) * ffn["x_k"]
-        k = torch.square(torch.relu(xk @ ffn["key"]["weight"].T))
+        k = xk @ ffn["key"]["weight"].T
+        k = ops.rwkv7_relusq(k) if cls.fuse_mix else torch.square(torch.relu(k))
         return k @ ffn["value"]["weight"].T, x[torch.arange(x.shape[0], device=x.device), last_idx]
 
     @classmethod

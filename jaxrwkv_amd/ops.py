@@ -522,6 +522,38 @@ def rwkv7_agate(x, a0):
     return _gate(x, a0, 1)
 
 
+def _relusq_fwd(x):
+    out = torch.empty_like(x)
+    rc = _lib.load().hiprwkv_rwkv7_relusq(_stream(), _DT[x.dtype], x.numel(), _p(x), _p(out))
+    _lib.check(rc, "hiprwkv_rwkv7_relusq")
+    return out
+
+
+class _ReluSq(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, x):
+        ctx.save_for_backward(x)
+        return _relusq_fwd(x)
+
+    @staticmethod
+    def backward(ctx, g):
+        x, = ctx.saved_tensors
+        g = _dev(g, x.dtype)
+        dx = torch.empty_like(x)
+        rc = _lib.load().hiprwkv_rwkv7_relusq_bwd(_stream(), _DT[x.dtype], x.numel(), _p(x), _p(g), _p(dx))
+        _lib.check(rc, "hiprwkv_rwkv7_relusq_bwd")
+        return dx
+
+
+def rwkv7_relusq(x):
+    """Channel mixing's activation, rwkv7.py:196: ``relu(x)**2`` in one pass; differentiable.  numel a multiple of 8."""
+    assert x.numel() % 8 == 0, x.shape
+    x = _dev(x, x.dtype)
+    if torch.is_grad_enabled() and x.requires_grad:
+        return _ReluSq.apply(x)
+    return _relusq_fwd(x)
+
+
 def _vmix_fwd(v, vf, x, v0):
     lib = _lib.load()
     io = v.dtype

@@ -101,6 +101,8 @@ def test_misaligned_pointers_are_refused_by_every_entry_point():
     assert lib.hiprwkv_rwkv7_decay_bwd(null, 1, 8, 64, ok, ok, ok, ok, null) == -1 and b"null" in msg()
     assert lib.hiprwkv_rwkv7_agate(null, 7, 8, 64, ok, ok, ok) == -1 and b"dtype" in msg()
     assert lib.hiprwkv_rwkv7_agate_bwd(null, 1, 0, 64, ok, ok, ok, ok, ok) == -1 and b"positive" in msg()
+    assert lib.hiprwkv_rwkv7_relusq(null, 1, 60, ok, ok) == -1 and b"multiple of 8" in msg()
+    assert lib.hiprwkv_rwkv7_relusq_bwd(null, 1, 64, ok, bad, ok) == -1 and b"aligned" in msg()
     assert lib.hiprwkv_rwkv7_vmix(null, 1, 8, 64, ok, ok, ok, ok, bad) == -1 and b"aligned" in msg()
     assert lib.hiprwkv_rwkv7_vmix_bwd(null, 1, 8, 64, ok, ok, ok, ok, ok, ok, bad, ok, ok) == -1 and b"aligned" in msg()
     # token shift + interpolation: pointer arrays in host memory, C a multiple of 8, one or six outputs

@@ -271,7 +271,7 @@ def test_token_shift_interpolation_forward_and_backward_against_torch(dtype, n_o
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("shape", [(3, 37, 128), (1, 1, 64), (2, 300, 2048 + 64)])
 def test_decay_value_mix_and_gate_forward_and_backward_against_torch(dtype, shape):
-    """ops.rwkv7_decay / rwkv7_vmix / rwkv7_agate (rwkv7.py:237, :241-242, :244), values and all cotangents, against
+    """ops.rwkv7_decay / rwkv7_vmix / rwkv7_agate / rwkv7_relusq (rwkv7.py:237, :241-242, :244, :196), values and all cotangents, against
     torch autograd of the plain formulas in fp32 on the same (dtype-rounded) inputs."""
     from jaxrwkv_amd import ops
     B, T, C = shape
@@ -284,6 +284,7 @@ def test_decay_value_mix_and_gate_forward_and_backward_against_torch(dtype, shap
         "decay": (lambda x_, p_: ops.rwkv7_decay(x_, p_),
                   lambda x_, p_: -torch.nn.functional.softplus(-(p_.float() + x_.float())) - 0.5, (x, p)),
         "agate": (lambda x_, p_: ops.rwkv7_agate(x_, p_), lambda x_, p_: torch.sigmoid(p_.float() + x_.float()), (x, p)),
+        "relusq": (lambda x_: ops.rwkv7_relusq(x_), lambda x_: torch.square(torch.relu(x_.float())), (x,)),
         # every input converted once: its cotangent is then rounded to the input's dtype once, as in the kernel
         "vmix": (lambda v_, f_, x_, p_: ops.rwkv7_vmix(v_, f_, x_, p_),
                  lambda v_, f_, x_, p_: (lambda v32: v32 + (f_.float() - v32) * torch.sigmoid(p_.float() + x_.float()))(v_.float()),
