@@ -84,6 +84,17 @@ __device__ __forceinline__ bool wait_ready_peeked(SyncN<NC>* sy, int slot, int w
   return wait_ready(sy, slot, want);
 }
 
+// Buffer addressing for the consumers' per-token scalars (2- and 4-byte accesses at (token 4g+i, element 16q+n)): a
+// descriptor on the uniform base of the chunk (scalar registers), the lane's byte offset in one vector register and
+// the token's offset as a scalar operand, so that no access costs vector address arithmetic or a register pair.
+// Measured on the same box: it takes 2 % off the WKV7 reverse sweep C (16 loads and 12 stores per consumer and chunk)
+// and is used there only: with it the sweeps whose consumers just store were no faster (WKV6) or 1.5-2.7 % slower
+// (WKV7 sweeps A and B).
+using rsrc_t = __amdgpu_buffer_rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void* base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7fffffff, 0x00020000);
+}
+
 // Test hook (HIPRWKV_DEBUG_DROP_PUBLISH): the producer of the last step does not publish it, so that the consumers'
 // bounded wait runs out while every wave still ends normally.
 constexpr unsigned FLAG_DROP_PUBLISH = 0x100u;

@@ -327,16 +327,18 @@ struct Cursor {
 };
 
 __device__ __forceinline__ void prefetch(Pre& p, const Cursor& cu, int nvalid, int g) {
-  const size_t lo = (size_t)cu.voff;
+  const rsrc_t rf = make_rsrc(cu.ef), rk = make_rsrc(cu.k), rb = make_rsrc(cu.b), rw = make_rsrc(cu.w);
+  const int o2 = (int)(cu.voff * 2u), o4 = (int)(cu.voff * 4u);
+  const int tok = (int)cu.tok_bytes;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     float f = 0.f;
     uint16_t k = 0, b = 0, w = 0;
     if (nvalid == CK || 4 * g + i < nvalid) {      // the first test is uniform: no lane predicate but in a partial chunk
-      f = *reinterpret_cast<const float*>(cu.ef + lo * 4 + 2 * i * cu.tok_bytes);
-      k = *reinterpret_cast<const uint16_t*>(cu.k + lo * 2 + i * cu.tok_bytes);
-      b = *reinterpret_cast<const uint16_t*>(cu.b + lo * 2 + i * cu.tok_bytes);
-      w = *reinterpret_cast<const uint16_t*>(cu.w + lo * 2 + i * cu.tok_bytes);
+      f = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rf, o4, 2 * i * tok, 0));
+      k = __builtin_amdgcn_raw_buffer_load_b16(rk, o2, i * tok, 0);
+      b = __builtin_amdgcn_raw_buffer_load_b16(rb, o2, i * tok, 0);
+      w = __builtin_amdgcn_raw_buffer_load_b16(rw, o2, i * tok, 0);
     }
     p.f[i] = f;
     p.k[i] = k; p.b[i] = b; p.w[i] = w;
@@ -487,12 +489,13 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
   __builtin_amdgcn_sched_barrier(0);
   if (has_next) prefetch(pre_next, cu_next, CK, g);
   __builtin_amdgcn_sched_barrier(0);
-  const size_t lo = (size_t)cu.voff;
+  const rsrc_t rgk = make_rsrc(cu.gk), rgb = make_rsrc(cu.gb), rgw = make_rsrc(cu.gw);
+  const int o2 = (int)(cu.voff * 2u), tokb = (int)cu.tok_bytes;
   auto put = [&](int i, bool full) {
     if (full || 4 * g + i < nvalid) {
-      *reinterpret_cast<uint16_t*>(cu.gk + lo * 2 + i * cu.tok_bytes) = ok[i];
-      *reinterpret_cast<uint16_t*>(cu.gb + lo * 2 + i * cu.tok_bytes) = ob[i];
-      *reinterpret_cast<uint16_t*>(cu.gw + lo * 2 + i * cu.tok_bytes) = ow[i];
+      __builtin_amdgcn_raw_buffer_store_b16(ok[i], rgk, o2, i * tokb, 0);
+      __builtin_amdgcn_raw_buffer_store_b16(ob[i], rgb, o2, i * tokb, 0);
+      __builtin_amdgcn_raw_buffer_store_b16(ow[i], rgw, o2, i * tokb, 0);
     }
   };
   if (nvalid == CK) {
