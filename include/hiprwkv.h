@@ -129,6 +129,18 @@ int hiprwkv_wkv6_fwd(hiprwkv_stream stream, int io_dtype, int state_dtype,
                      const uint32_t* length, const uint8_t* new_starts,
                      void* out, void* new_s, unsigned flags);
 
+/* hiprwkv_wkv6_fwd for a decode step (T <= HIPRWKV_SMALL_T) on a state inside the reference's packed model state
+ * (rwkv6.py:148-153 default_state: (L, 2+N, C) per sequence; :221-224 the slice state[1:] of the time-mixing part,
+ * reshaped to (H,N,N) around inner_loop and written back): `s` and `new_s` point at the first sequence's state, the
+ * states of consecutive sequences are `*_batch_stride` elements apart (>= H*N*N, a multiple of 16 bytes); `new_s` may
+ * be `s` for an update in place.  Same conventions as hiprwkv_wkv7_step. */
+int hiprwkv_wkv6_step(hiprwkv_stream stream, int io_dtype, int state_dtype,
+                      int64_t B, int64_t T, int64_t H, int64_t N,
+                      const void* r, const void* k, const void* v, const void* w,
+                      const void* u, const void* s, int64_t s_batch_stride,
+                      const uint32_t* length, const uint8_t* new_starts,
+                      void* out, void* new_s, int64_t new_s_batch_stride, unsigned flags);
+
 size_t hiprwkv_wkv6_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t N);
 
 /* Cotangents of wkv6_fwd: gr,gk,gv,gw (B,T,H,N) io_dtype; gu (B,H,N) fp32, to be summed

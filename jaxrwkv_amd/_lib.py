@@ -30,6 +30,8 @@ SIGNATURES = {
     "hiprwkv_wkv7_bwd": (_int, [_vp, _int, _int, _i64, _i64, _i64, _i64] + [_vp] * 7 + [_vp, _vp] + [_vp] * 3
                          + [_vp] * 7 + [_vp, _sz, _u32]),
     "hiprwkv_wkv6_fwd": (_int, [_vp, _int, _int, _i64, _i64, _i64, _i64] + [_vp] * 6 + [_vp, _vp] + [_vp, _vp, _u32]),
+    "hiprwkv_wkv6_step": (_int, [_vp, _int, _int, _i64, _i64, _i64, _i64] + [_vp] * 5 + [_vp, _i64] + [_vp, _vp]
+                          + [_vp, _vp, _i64, _u32]),
     "hiprwkv_wkv6_bwd_workspace_bytes": (_sz, [_i64] * 4),
     "hiprwkv_wkv6_bwd": (_int, [_vp, _int, _int, _i64, _i64, _i64, _i64] + [_vp] * 6 + [_vp, _vp] + [_vp, _vp]
                          + [_vp] * 6 + [_vp, _sz, _u32]),

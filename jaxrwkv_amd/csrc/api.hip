@@ -94,7 +94,7 @@ unsigned* status_word() {
 extern "C" {
 
 const char* hiprwkv_last_error(void) { return g_err; }
-int hiprwkv_version(void) { return 106; }
+int hiprwkv_version(void) { return 107; }
 
 int hiprwkv_handshake_failures(hiprwkv_stream stream, unsigned* count) {
   if (count == nullptr) return fail(HIPRWKV_EINVAL, "handshake_failures: null count pointer");
@@ -242,6 +242,38 @@ int hiprwkv_wkv6_fwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64
   hipStream_t st = static_cast<hipStream_t>(stream);
   hipError_t e = small_t ? launch_wkv6_small_t_fwd(A, st) : chunked ? launch_wkv6_chunk_fwd(A, st) : launch_wkv6_seq_fwd(A, st);
   if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "wkv6_fwd: %s", hipGetErrorString(e));
+  return HIPRWKV_OK;
+}
+
+int hiprwkv_wkv6_step(hiprwkv_stream stream, int io_dtype, int state_dtype, int64_t B, int64_t T, int64_t H, int64_t N,
+                      const void* r, const void* k, const void* v, const void* w, const void* u, const void* s,
+                      int64_t s_batch_stride, const uint32_t* length, const uint8_t* new_starts, void* out, void* new_s,
+                      int64_t new_s_batch_stride, unsigned flags) {
+  int rc = check_matrix_shape("wkv6_step", io_dtype, state_dtype, B, T, H, N);
+  if (rc) return rc;
+  if (T > HIPRWKV_SMALL_T) return fail(HIPRWKV_EINVAL, "wkv6_step: T=%lld, at most %d tokens per call", (long long)T, HIPRWKV_SMALL_T);
+  const void* req[] = {r, k, v, w, u, s, out, new_s};
+  for (const void* p : req) {
+    if (p == nullptr) return fail(HIPRWKV_EINVAL, "wkv6_step: null tensor pointer");
+    if (!aligned16(p)) return fail(HIPRWKV_EINVAL, "wkv6_step: tensor pointers must be 16-byte aligned");
+  }
+  const int64_t dense = H * N * N;
+  const int64_t elem = state_dtype == HIPRWKV_F32 ? 4 : 2;
+  for (int64_t stride : {s_batch_stride, new_s_batch_stride}) {
+    if (stride < dense) return fail(HIPRWKV_EINVAL, "wkv6_step: state batch stride %lld is less than H*N*N = %lld", (long long)stride, (long long)dense);
+    if ((stride * elem) % 16 != 0) return fail(HIPRWKV_EINVAL, "wkv6_step: state batch stride must be a multiple of 16 bytes");
+  }
+  Wkv6Args A;
+  memset(&A, 0, sizeof(A));
+  A.B = B; A.T = T; A.H = H;
+  A.r = r; A.k = k; A.v = v; A.w = w; A.u = u; A.s = s;
+  A.length = length; A.ns = new_starts;
+  A.out = out; A.new_s = new_s;
+  A.io_f32 = io_dtype == HIPRWKV_F32; A.st_f32 = state_dtype == HIPRWKV_F32;
+  A.flags = flags;
+  A.s_bstride = s_batch_stride; A.new_s_bstride = new_s_batch_stride;
+  const hipError_t e = launch_wkv6_small_t_fwd(A, static_cast<hipStream_t>(stream));
+  if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "wkv6_step: %s", hipGetErrorString(e));
   return HIPRWKV_OK;
 }
 

@@ -34,7 +34,13 @@ __global__ __launch_bounds__(256) void wkv6_small_t_kernel(Wkv6Args A) {
   const uint8_t* ns = A.ns ? A.ns + b * A.T : nullptr;
   // the returned state is the reset state there (associative-scan rule)
   const bool q2drop = (A.flags & 1u) && L < A.T && ns != nullptr && ns[L] != 0;
-  const size_t sel = (((size_t)b * A.H + h) * 64 + c0) * 64 + j;
+  // a sequence's state is H*64*64 contiguous elements; consecutive sequences may lie further apart (a layer's rows of
+  // a packed model state).  Every thread reads its 16 elements once, up front, and writes them once: s and new_s may
+  // be the same memory.
+  const size_t in_head = ((size_t)h * 64 + c0) * 64 + j;
+  const size_t dense = (size_t)A.H * 4096;
+  const size_t sel = (size_t)b * (A.s_bstride ? (size_t)A.s_bstride : dense) + in_head;
+  const size_t sel_out = (size_t)b * (A.new_s_bstride ? (size_t)A.new_s_bstride : dense) + in_head;
   float S[16], u[16];
   {
     const ST* p = reinterpret_cast<const ST*>(A.s) + sel;
@@ -42,7 +48,7 @@ __global__ __launch_bounds__(256) void wkv6_small_t_kernel(Wkv6Args A) {
     for (int c = 0; c < 16; ++c) S[c] = ld_f(p + (size_t)c * 64);
   }
   ld16<IO>(A.u, (size_t)h * 64 + c0, u);
-  if (L == 0) st_col<ST>(A.new_s, sel, S, q2drop);
+  if (L == 0) st_col<ST>(A.new_s, sel_out, S, q2drop);
   for (int64_t t = 0; t < A.T; ++t) {
     const size_t tel = (((size_t)b * A.T + t) * A.H + h) * 64;
     float w[16], r[16], k[16];
@@ -68,7 +74,7 @@ __global__ __launch_bounds__(256) void wkv6_small_t_kernel(Wkv6Args A) {
     }
     const float y = quad_sum(y0 + y1);
     if (q == 0) st_f(reinterpret_cast<IO*>(A.out) + tel + j, y);
-    if (t == L - 1) st_col<ST>(A.new_s, sel, S, q2drop);
+    if (t == L - 1) st_col<ST>(A.new_s, sel_out, S, q2drop);
   }
 }
 

@@ -49,6 +49,9 @@ struct Wkv6Args {
   float* er;   // workspace (B,T,H,64): r . (S' dy)
   float* eI;   // workspace (B,H,64): rowsum(dS_out * S_{length-1})
   unsigned* status;   // device word counting workgroups whose hand-shake gave up (may be null)
+  // Elements between the states of consecutive sequences in `s` / `new_s`; 0 = dense (H*64*64).  Honoured by the
+  // small-T kernel only (states read and written inside a packed model state).
+  int64_t s_bstride, new_s_bstride;
 };
 
 // Wkv4Args::flags bit: the workspace already holds the checkpoints (HIPRWKV_CKPT_READY)

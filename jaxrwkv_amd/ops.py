@@ -195,6 +195,29 @@ def wkv6_fwd(r, k, v, w, u, s, length=None, new_starts=None, compat=True, force_
     return new_s, y
 
 
+def wkv6_step(r, k, v, w, u, s, new_s, length=None, new_starts=None, compat=True):
+    """A decode step (T <= 8) on states inside a packed model state: ``s`` and ``new_s`` are views with a batch axis in
+    front and H*N*N contiguous elements per sequence (rwkv6.py:221-224); ``new_s`` is written in place (it may be
+    ``s``).  ``w`` (B,T,H,N) or the shared (H,N) decay.  Returns y.  No autograd."""
+    lib = _lib.load()
+    io = r.dtype
+    B, T, H, N = r.shape
+    r, k, v = (_dev(x, io) for x in (r, k, v))
+    per_head = w.numel() == H * N and (B * T != 1 or w.dim() == 2)
+    w = _dev(w.reshape(H, N) if per_head else w.reshape(B, T, H, N), io)
+    u = _dev(u.reshape(H, N), io)
+    s, s_stride = _packed_state(s, B, H, N)
+    new_s, ns_stride = _packed_state(new_s, B, H, N)
+    assert s.dtype == new_s.dtype
+    length, new_starts = _length_ns(length, new_starts, B, T, r.device)
+    y = torch.empty_like(r)
+    flags = _flags(compat, False, True, 0) | (_lib.W_PER_HEAD if per_head else 0)
+    rc = lib.hiprwkv_wkv6_step(_stream(), _DT[io], _DT[s.dtype], B, T, H, N, _p(r), _p(k), _p(v), _p(w), _p(u), _p(s),
+                               s_stride, _p(length), _p(new_starts), _p(y), _p(new_s), ns_stride, flags)
+    _lib.check(rc, "hiprwkv_wkv6_step")
+    return y
+
+
 def wkv6_bwd(r, k, v, w, u, s, length, new_starts, gy, gs_out=None, compat=True, force_seq=False, debug_flags=0):
     """Cotangents (gr, gk, gv, gw, gu, gs) of ``wkv6_fwd``; gu is summed over the batch here, and so is gw over batch
     and tokens when ``w`` is the shared (H,N) decay.

@@ -27,3 +27,11 @@ class HipRWKV:
         if not batched:
             new_s, y = new_s[0], y[0]
         return new_s, y
+
+    @classmethod
+    def step_packed(cls, r, k, v, w, time_first, s, new_s, length, new_starts):
+        """``inner_loop`` for a few tokens (T <= 8, decode) with the state read from and written to views of the packed
+        model state (``state[:, layer, 2:]`` with a batch axis in front, rwkv6.py:221-224) instead of copies of them;
+        batched, no autograd.  Returns ``out``; ``new_s`` is filled in place."""
+        return ops.wkv6_step(r, k, v, w.reshape(r.shape), time_first.reshape(r.shape[2], r.shape[3]), s, new_s, length,
+                             new_starts, cls.assoc_compat)

@@ -66,6 +66,10 @@ def test_argument_validation_without_gpu():
     assert step(1, 8191, 8192) == -1 and b"less than" in lib.hiprwkv_last_error()
     assert step(1, 8192, 8192 + 4) == -1 and b"16 bytes" in lib.hiprwkv_last_error()
     assert step(1, 8192 + 2, 8192, st=0) == -1 and b"16 bytes" in lib.hiprwkv_last_error()
+    step6 = lambda T, s_stride, o_stride: lib.hiprwkv_wkv6_step(null, 1, 1, 2, T, 2, 64, *([ok] * 6), s_stride, null, null, ok,
+                                                                ok, o_stride, 0)
+    assert step6(9, 8192, 8192) == -1 and b"at most 8" in lib.hiprwkv_last_error()
+    assert step6(1, 8192, 100) == -1 and b"less than" in lib.hiprwkv_last_error()
     assert lib.hiprwkv_wkv6_bwd_workspace_bytes(2, 16, 2, 64) >= 2 * 16 * 2 * 64 * 4
 
 

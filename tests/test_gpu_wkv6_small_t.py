@@ -94,3 +94,37 @@ def test_decode_steps_equal_one_prefill_call():
     torch.cuda.synchronize()
     assert_close("y", host(torch.cat(ys, 1)), host(y_full))
     assert_close("state", host(s), host(s_full))
+
+
+@pytest.mark.parametrize("io,st", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                   (torch.bfloat16, torch.float32)])
+@pytest.mark.parametrize("T", [1, 3])
+def test_step_on_a_packed_model_state_equals_the_dense_call(io, st, T):
+    """hiprwkv_wkv6_step reads and writes a layer's rows of a (B, L, 2+N, C) model state in place (rwkv6.py:148-153,
+    221-224): same bits as the dense call on copies of those rows, nothing else of the new model state touched, and an
+    update in place (new_s = s) gives the same again."""
+    from jaxrwkv_amd import ops
+    B, H, N, L, layer = 3, 2, 64, 3, 1
+    C = H * N
+    x = wkv6_inputs(B, T, H, N, seed=500 + T, bf16=(io == torch.bfloat16), p_reset=0.3)
+    x["length"][0] = 0
+    t = {n: dev(x[n], io) for n in ("r", "k", "v", "w", "u")}
+    length, ns = dev(x["length"]), dev(x["new_starts"])
+    g = torch.Generator(device="cuda").manual_seed(7)
+    state = (0.1 * torch.randn((B, L, 2 + N, C), device="cuda", generator=g)).to(st)
+    new_state = torch.full_like(state, 7.0)
+    dense = state[:, layer, 2:].reshape(B, H, N, N).contiguous()
+    ref_s, ref_y = ops.wkv6_fwd(t["r"], t["k"], t["v"], t["w"], t["u"], dense, length, ns)
+    y = ops.wkv6_step(t["r"], t["k"], t["v"], t["w"], t["u"], state[:, layer, 2:], new_state[:, layer, 2:], length, ns)
+    torch.cuda.synchronize()
+    assert torch.equal(y, ref_y)
+    assert torch.equal(new_state[:, layer, 2:].reshape(B, H, N, N), ref_s)
+    untouched = torch.ones_like(new_state, dtype=torch.bool)
+    untouched[:, layer, 2:] = False
+    assert bool((new_state[untouched] == 7.0).all())
+    work = state.clone()
+    y2 = ops.wkv6_step(t["r"], t["k"], t["v"], t["w"], t["u"], work[:, layer, 2:], work[:, layer, 2:], length, ns)
+    torch.cuda.synchronize()
+    assert torch.equal(y2, ref_y)
+    assert torch.equal(work[:, layer, 2:].reshape(B, H, N, N), ref_s)
+    assert torch.equal(work[untouched], state[untouched])
