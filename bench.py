@@ -29,18 +29,22 @@ B, T, H, N = 8, 4096, 32, 64
 # figures in profiles/), each with the sha1 prefix of the kernel source it was measured on: when the source has
 # changed since, `roofline.traffic` is null instead of a stale figure.
 MEASURED_TRAFFIC = {
-    "wkv7_fwd": (948.5e6, "wkv7_fwd.hip", "86253aea7c44"),
-    "wkv4_fwd": (4028.7e6, "wkv4.hip", "d83a0992a92e"),
-    "wkv6_fwd": (688.5e6, "wkv6_fwd.hip", "0a029503ae09"),
+    "wkv7_fwd": (948.5e6, "wkv7_fwd.hip", "SHA_WKV7", "profiles/wkv7_fwd_B8_T4096_H32_bf16.md"),
+    "wkv4_fwd": (4028.7e6, "wkv4.hip", "d83a0992a92e", "profiles/wkv4_fwd_B32_T4096_C2560_f32.md"),
+    "wkv6_fwd": (688.5e6, "wkv6_fwd.hip", "SHA_WKV6", "profiles/wkv6_fwd_bwd_B16_T2048_H32_bf16.md"),
 }
 
 
 def measured_traffic(name):
+    """(bytes, source) of the counter run recorded in profiles/: `roofline.traffic` is NOT measured by this run, it
+    is the figure of the named profile, given only while the kernel source still has the hash it was measured on."""
     import hashlib
-    nbytes, src, sha = MEASURED_TRAFFIC[name]
+    nbytes, src, sha, profile = MEASURED_TRAFFIC[name]
     path = os.path.join(ROOT, "jaxrwkv_amd", "csrc", src)
     now = hashlib.sha1(open(path, "rb").read()).hexdigest()[:12]
-    return nbytes if sha == now else None
+    if sha != now:
+        return None, f"{profile} (stale: {src} has changed since the counter run)"
+    return nbytes, f"{profile} (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, not measured by this run)"
 
 
 def make_inputs(torch, seed=0):
@@ -177,8 +181,54 @@ def stream_probe(torch):
 
 def roofline(bytes_per_launch, kern_ms, traffic):
     achieved = bytes_per_launch / (kern_ms * 1e-3) / 1e9
+    nbytes, source = traffic if traffic is not None else (None, None)
     return {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": achieved / HBM_PEAK_GBS,
-            "traffic": traffic, "kernel_ms": kern_ms, "algorithmic_bytes": bytes_per_launch}
+            "traffic": nbytes, "traffic_source": source, "kernel_ms": kern_ms, "algorithmic_bytes": bytes_per_launch}
+
+
+def power_probe(torch, fn, seconds=1.6):
+    """Socket power while `fn` runs back to back: launches are queued for about `seconds`, `amd-smi` is read twice
+    while the GPU works through them.  None where the tool is missing or prints nothing usable."""
+    import shutil
+    import subprocess
+    if shutil.which("amd-smi") is None:
+        return None
+
+    def read(args, key):
+        try:
+            txt = subprocess.run(["amd-smi"] + args, capture_output=True, text=True, timeout=20).stdout
+        except Exception:
+            return None
+        for line in txt.splitlines():
+            if key in line:
+                try:
+                    return float(line.split(":")[1].split()[0])
+                except (IndexError, ValueError):
+                    return None
+        return None
+
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(20):
+        fn()
+    torch.cuda.synchronize()
+    e0.record()
+    for _ in range(5):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    per_call = e0.elapsed_time(e1) / 5 * 1e-3
+    for _ in range(max(10, int(seconds / per_call))):
+        fn()
+    time.sleep(0.5)
+    w1 = read(["metric", "-g", "0", "--power"], "SOCKET_POWER")
+    w2 = read(["metric", "-g", "0", "--power"], "SOCKET_POWER")
+    busy = not torch.cuda.current_stream().query()
+    torch.cuda.synchronize()
+    cap = read(["static", "-g", "0", "--limit"], "MAX_POWER")
+    if w1 is None and w2 is None:
+        return None
+    return {"socket_w": [w1, w2], "cap_w": cap, "gpu_still_busy_after_reads": busy,
+            "how": "amd-smi metric --power, read twice while the forward kernel runs back to back"}
 
 
 def bench_wkv7(torch, ops, args):
@@ -204,12 +254,12 @@ def bench_wkv7(torch, ops, args):
                                         x["new_starts"], compat=True, want_sa=True, force_seq=args.seq)
             return ops.wkv7_bwd(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], x["length"], x["new_starts"],
                                 x["dy"], sa, None, compat=True, force_seq=args.seq)
-        n2 = max(2, args.steps // 4)
-        wall2, _ = time_region(torch, fwd_bwd, n2, 1)
+        n2 = max(10, args.steps // 4)
+        wall2, _ = time_region(torch, fwd_bwd, n2, 2)
         ms2 = 1e3 * wall2 / n2
         # forward (7 tensors) + backward reads r,w,k,v,a,b,dy and writes 6 gradients: 20 token tensors in bf16
         fb_bytes = 20 * tokens * H * N * 2 + 4 * B * H * N * N * 4
-        out["fwd_bwd"] = {"tokens_per_s": tokens / (ms2 * 1e-3), "ms_per_step": ms2,
+        out["fwd_bwd"] = {"tokens_per_s": tokens / (ms2 * 1e-3), "ms_per_step": ms2, "steps": n2, "warmup": 2,
                           "hbm_frac": fb_bytes / (ms2 * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": fb_bytes,
                           "note": "forward keeps the residual sa (fp16 beside bf16 I/O); backward = three sweeps (reverse, forward, reverse), " +
                                   ("sequential fp32 VALU kernels" if args.seq else "chunked MFMA kernels") +
@@ -230,6 +280,8 @@ def bench_wkv7(torch, ops, args):
                           "mfma_frac": None if args.seq else fp32_mfma_flops(tokens) / (k32 * 1e-3) / 1e12 / 157.3,
                           "kernel": "sequential fp32 VALU" if args.seq else "chunked, v_mfma_f32_16x16x4_f32 (fp32 operands)"}
         del x32
+    if not args.no_power:
+        out["power"] = power_probe(torch, fwd)
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
         out["cpu_baseline_sequential"] = cpu_baseline_sequential()
@@ -261,12 +313,13 @@ def bench_wkv6(torch, ops, args):
     out = base_record("WKV6 fwd tokens/s (B16 T2048 H32 N64 bf16)", tokens / (ms_step * 1e-3), ms_step, args, "bf16",
                       "isolated WKV6 op, B=16 T=2048 H=32 N=64 bf16, zero state, new_starts~Bernoulli(1/512) "
                       "(BASELINE configs[2])",
-                      {"kernel": "chunked MFMA forward and backward (bf16 hi+lo operands, fp32 accumulate)"})
+                      {"kernel": "chunked MFMA; forward on fp16 operands (bf16 pairs in the Gram tile), backward sweeps on "
+                                 "bf16 hi+lo pairs; fp32 state and accumulation"})
     out["roofline"] = roofline(fwd_bytes, kern_ms, measured_traffic("wkv6_fwd"))
     if not args.no_bwd:
         fb = lambda: ops.wkv6_bwd(r, k, v, w, u, s, None, ns, dy, None, compat=True)
-        n2 = max(2, args.steps // 4)
-        wall2, _ = time_region(torch, lambda: (fwd(), fb()), n2, 1)
+        n2 = max(10, args.steps // 4)
+        wall2, _ = time_region(torch, lambda: (fwd(), fb()), n2, 2)
         ms2 = 1e3 * wall2 / n2
         fb_bytes = 14 * tokens * H * N * 2 + 4 * b6 * H * N * N * 4
         out["fwd_bwd"] = {"tokens_per_s": tokens / (ms2 * 1e-3), "ms_per_step": ms2,
@@ -297,8 +350,8 @@ def bench_wkv4(torch, ops, args):
     if not args.no_bwd:
         gy = f(g.standard_normal((b4, t4, c4), dtype=np.float32))
         bwd = lambda: ops.wkv4_bwd(w, u, k, v, s, length, None, gy, None, compat=True)
-        n2 = max(2, args.steps // 4)
-        wall2, kern2 = time_region(torch, bwd, n2, 1)
+        n2 = max(10, args.steps // 4)
+        wall2, kern2 = time_region(torch, bwd, n2, 2)
         # backward alone: reads k, v, gy and writes gk, gv (fp32)
         bwd_bytes = 5 * tokens * c4 * 4
         out["bwd"] = {"ms_per_call": kern2, "hbm_frac": bwd_bytes / (kern2 * 1e-3) / 1e9 / HBM_PEAK_GBS,
@@ -309,7 +362,7 @@ def bench_wkv4(torch, ops, args):
         def fwd_bwd():
             _, _, ck = ops.wkv4_fwd(w, u, k, v, s, length, None, compat=True, want_ckpt=True)
             return ops.wkv4_bwd(w, u, k, v, s, length, None, gy, None, compat=True, ckpt=ck)
-        _, kern3 = time_region(torch, fwd_bwd, n2, 1)
+        _, kern3 = time_region(torch, fwd_bwd, n2, 2)
         fb_bytes = fwd_bytes + bwd_bytes
         out["fwd_bwd"] = {"ms_per_step": kern3, "tokens_per_s": tokens / (kern3 * 1e-3),
                           "hbm_frac": fb_bytes / (kern3 * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": fb_bytes,
@@ -404,6 +457,9 @@ def main():
     ap.add_argument("--no-bwd", action="store_true")
     ap.add_argument("--no-fp32", action="store_true", help="WKV7: skip the fp32-I/O leg")
     ap.add_argument("--seq", action="store_true", help="WKV7: force the sequential fp32 VALU kernel")
+    ap.add_argument("--no-power", action="store_true", help="WKV7: skip the socket-power reading (amd-smi)")
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="WKV7: skip the compact WKV6 / WKV4 records appended to the line")
     ap.add_argument("--no-stream-probe", action="store_true",
                     help="skip the streaming-bandwidth probe (three 1 GiB arrays) that is reported beside the roofline")
     ap.add_argument("--copy-probe", action="store_true",
@@ -427,6 +483,18 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     out = {"wkv7": bench_wkv7, "wkv6": bench_wkv6, "wkv4": bench_wkv4, "model7": bench_model7}[args.workload](torch, ops, args)
+    if args.workload == "wkv7" and not args.no_secondary:
+        # the two secondary ops under the same clock: forward time and roofline fraction, forward+backward beside it
+        sub = argparse.Namespace(**vars(args))
+        sub.steps, sub.warmup = max(20, args.steps // 2), max(3, args.warmup // 2)
+        for name, fn in (("wkv6", bench_wkv6), ("wkv4", bench_wkv4)):
+            full = fn(torch, ops, sub)
+            torch.cuda.empty_cache()
+            out[name] = {"workload": full["config"]["workload"], "fwd_ms": full["roofline"]["kernel_ms"],
+                         "fwd_tokens_per_s": full["value"], "fwd_hbm_frac": full["roofline"]["frac"],
+                         "steps": sub.steps, "warmup": sub.warmup,
+                         "fwd_bwd_ms": full.get("fwd_bwd", {}).get("ms_per_step"),
+                         "fwd_bwd_hbm_frac": full.get("fwd_bwd", {}).get("hbm_frac")}
     if not args.no_stream_probe:
         out["roofline"]["stream_probe"] = stream_probe(torch)
     print(json.dumps(out))

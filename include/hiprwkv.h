@@ -60,6 +60,9 @@ extern "C" {
  * consumer waves' wait runs out (a few milliseconds), every wave still ends normally, the outputs of every
  * (sequence, head) are NaN and hiprwkv_handshake_failures() has advanced by B*H per kernel. */
 #define HIPRWKV_DEBUG_DROP_PUBLISH 0x100u
+/* Every flag a production caller may pass.  Entry points refuse other bits, and refuse HIPRWKV_DEBUG_DROP_PUBLISH
+ * unless the process runs with HIPRWKV_ENABLE_DEBUG_FLAGS=1 in its environment. */
+#define HIPRWKV_PUBLIC_FLAGS (HIPRWKV_COMPAT_ASSOC | HIPRWKV_FORCE_SEQ | HIPRWKV_NO_SMALL_T | HIPRWKV_W_PER_HEAD | HIPRWKV_CKPT_READY)
 
 typedef void* hiprwkv_stream; /* a hipStream_t */
 
@@ -72,6 +75,22 @@ int hiprwkv_version(void);
  * device to *count (host memory).  Unlike every other entry point it synchronises `stream`.  No counterpart in
  * the reference; for health checks and tests. */
 int hiprwkv_handshake_failures(hiprwkv_stream stream, unsigned* count);
+
+/* Numeric events of the chunked matrix-core kernels since the process started, per device, copied to *count (host
+ * memory; synchronises `stream`).  Two things are counted, once per wave that meets them:
+ *  - a key channel whose log decay summed over a 16-token chunk is below -80 (a decay of e^-5 per token sustained over
+ *    the chunk; RWKV-7's own w <= -0.5 keeps it above -10): the chunked kernels, fp32 I/O included, scale that
+ *    channel's steps of the chunk to a total of -80, so its result is no longer exact.  Every sweep of a backward
+ *    call that meets such a chunk counts it again.  HIPRWKV_FORCE_SEQ has no such floor.
+ *  - inf or NaN in the carried state of the bf16-I/O forward kernels (WKV7, WKV6) after the last token: their matrix
+ *    operands are IEEE half, so |state|, |sa|, |v| or a decay-scaled input beyond 65504 overflow; y and the state
+ *    are then inf/NaN from that token on (until a reset starts a new state: an overflow whose state a later reset
+ *    discards shows in y alone).
+ * Magnitudes far below 1 lose precision silently instead: the half operands have 11 significant bits down to 6e-5
+ * and fewer below, so v (and with it the state and sa) scaled by 1e-5 doubles the error of y and 1e-7 brings it to
+ * 4 %; the op is linear in (v, s), so a caller with such values scales them by a power of two around the call.
+ * No counterpart in the reference; for health checks and tests. */
+int hiprwkv_numeric_events(hiprwkv_stream stream, unsigned* count);
 
 /* ---- WKV7 ------------------------------------------------------------------
  * Replaces ffi target "wkv7-fwd-{fp32,bf16}": operands w,r,k,v,a,b,s,length,new_starts

@@ -14,7 +14,8 @@ FORCE_SEQ = 2
 NO_SMALL_T = 4
 W_PER_HEAD = 0x10
 CKPT_READY = 0x20
-DEBUG_DROP_PUBLISH = 0x100
+DEBUG_DROP_PUBLISH = 0x100      # refused unless the process runs with HIPRWKV_ENABLE_DEBUG_FLAGS=1
+PUBLIC_FLAGS = COMPAT_ASSOC | FORCE_SEQ | NO_SMALL_T | W_PER_HEAD | CKPT_READY
 
 _vp, _i64, _int, _u32, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int, ctypes.c_uint, ctypes.c_size_t
 
@@ -23,6 +24,7 @@ SIGNATURES = {
     "hiprwkv_last_error": (ctypes.c_char_p, []),
     "hiprwkv_version": (_int, []),
     "hiprwkv_handshake_failures": (_int, [_vp, ctypes.POINTER(ctypes.c_uint)]),
+    "hiprwkv_numeric_events": (_int, [_vp, ctypes.POINTER(ctypes.c_uint)]),
     "hiprwkv_wkv7_fwd": (_int, [_vp, _int, _int, _i64, _i64, _i64, _i64] + [_vp] * 7 + [_vp, _vp] + [_vp, _vp, _vp, _u32]),
     "hiprwkv_wkv7_step": (_int, [_vp, _int, _int, _i64, _i64, _i64, _i64] + [_vp] * 6 + [_vp, _i64] + [_vp, _vp]
                           + [_vp, _vp, _i64, _u32]),

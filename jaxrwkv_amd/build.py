@@ -18,17 +18,33 @@ FLAGS = [
 ]
 
 
-def build(verbose=True):
+def build(verbose=True, jobs=None):
+    """Compiles every source to an object under ``jaxrwkv_amd/build/`` (in parallel) and links the shared library."""
+    from concurrent.futures import ThreadPoolExecutor
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + FLAGS + [os.path.join(CSRC, s) for s in SOURCES] + ["-o", LIB]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    out = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l)
-    if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + out)
-    if verbose and out.strip():
-        print(out)
+    objdir = os.path.join(HERE, "build")
+    os.makedirs(objdir, exist_ok=True)
+    compile_flags = [f for f in FLAGS if f != "-shared"]
+
+    def run(cmd):
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        out = "\n".join(l for l in res.stdout.splitlines() if "packed-fp32-ops" not in l)
+        if res.returncode != 0:
+            raise RuntimeError("hipcc failed:\n" + out)
+        if verbose and out.strip():
+            print(out)
+
+    def compile_one(src):
+        obj = os.path.join(objdir, os.path.splitext(src)[0] + ".o")
+        run([hipcc] + compile_flags + ["-c", os.path.join(CSRC, src), "-o", obj])
+        return obj
+
+    jobs = jobs or min(8, os.cpu_count() or 1)
+    with ThreadPoolExecutor(max_workers=jobs) as pool:
+        objs = list(pool.map(compile_one, SOURCES))
+    run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc"] + objs + ["-o", LIB])
     return LIB
 
 

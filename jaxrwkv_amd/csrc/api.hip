@@ -3,6 +3,7 @@
 
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <initializer_list>
@@ -38,9 +39,11 @@ int check_matrix_shape(const char* op, int io_dtype, int state_dtype, int64_t B,
 
 bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-// Counts the workgroups of the chunked kernels whose bounded hand-shake wait ran out (they overwrite their outputs
-// with NaN and add one here).  Every GPU holds its own copy of the word; its address is looked up once per device.
-__device__ unsigned int g_handshake_failures = 0u;
+// Word 0 counts the workgroups of the chunked kernels whose bounded hand-shake wait ran out (they overwrite their
+// outputs with NaN and add one here).  Word 1 counts numeric events of the chunked kernels: waves that had to cap a
+// channel's decay over a chunk, and waves that found inf or NaN in a carried state (an fp16 operand overflowed).
+// Every GPU holds its own copy of the words; their address is looked up once per device.
+__device__ unsigned int g_status_words[2] = {0u, 0u};
 
 constexpr int MAX_DEVICES = 64;
 std::mutex g_sym_mu;
@@ -75,6 +78,20 @@ void* scratch_base() {
   return g_scratch_ptr[dev];
 }
 
+// Public flag bits are accepted everywhere; the test hook HIPRWKV_DEBUG_DROP_PUBLISH only in a process that sets the
+// environment variable HIPRWKV_ENABLE_DEBUG_FLAGS=1, so that a stray bit cannot turn a production call's outputs
+// into NaN.  Unknown bits are refused.
+int check_flags(const char* op, unsigned flags) {
+  if (flags & ~(HIPRWKV_PUBLIC_FLAGS | HIPRWKV_DEBUG_DROP_PUBLISH))
+    return fail(HIPRWKV_EINVAL, "%s: unknown flag bits 0x%x", op, flags & ~(HIPRWKV_PUBLIC_FLAGS | HIPRWKV_DEBUG_DROP_PUBLISH));
+  if (flags & HIPRWKV_DEBUG_DROP_PUBLISH) {
+    static const bool enabled = [] { const char* e = getenv("HIPRWKV_ENABLE_DEBUG_FLAGS"); return e != nullptr && e[0] == '1'; }();
+    if (!enabled)
+      return fail(HIPRWKV_EINVAL, "%s: HIPRWKV_DEBUG_DROP_PUBLISH needs HIPRWKV_ENABLE_DEBUG_FLAGS=1 in the environment", op);
+  }
+  return HIPRWKV_OK;
+}
+
 // Address of the current device's failure counter, or null when it cannot be obtained (the kernels then skip the
 // count; the NaN poisoning does not depend on it).
 unsigned* status_word() {
@@ -83,7 +100,7 @@ unsigned* status_word() {
   std::lock_guard<std::mutex> lock(g_sym_mu);
   if (g_status_ptr[dev] == nullptr) {
     void* p = nullptr;
-    if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_handshake_failures)) != hipSuccess) return nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_status_words)) != hipSuccess) return nullptr;
     g_status_ptr[dev] = static_cast<unsigned*>(p);
   }
   return g_status_ptr[dev];
@@ -107,12 +124,24 @@ int hiprwkv_handshake_failures(hiprwkv_stream stream, unsigned* count) {
   return HIPRWKV_OK;
 }
 
+int hiprwkv_numeric_events(hiprwkv_stream stream, unsigned* count) {
+  if (count == nullptr) return fail(HIPRWKV_EINVAL, "numeric_events: null count pointer");
+  unsigned* word = status_word();
+  if (word == nullptr) return fail(HIPRWKV_ELAUNCH, "numeric_events: the device counter is not reachable");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  hipError_t e = hipMemcpyAsync(count, word + 1, sizeof(unsigned), hipMemcpyDeviceToHost, st);
+  if (e == hipSuccess) e = hipStreamSynchronize(st);
+  if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "numeric_events: %s", hipGetErrorString(e));
+  return HIPRWKV_OK;
+}
+
 int hiprwkv_wkv7_fwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64_t B, int64_t T, int64_t H, int64_t N,
                      const void* w, const void* r, const void* k, const void* v, const void* a, const void* b,
                      const void* s, const uint32_t* length, const uint8_t* new_starts, void* out, void* sa,
                      void* new_s, unsigned flags) {
   int rc = check_matrix_shape("wkv7_fwd", io_dtype, state_dtype, B, T, H, N);
   if (rc) return rc;
+  if ((rc = check_flags("wkv7_fwd", flags)) != HIPRWKV_OK) return rc;
   const void* req[] = {w, r, k, v, a, b, s, out, new_s};
   for (const void* p : req) {
     if (p == nullptr) return fail(HIPRWKV_EINVAL, "wkv7_fwd: null tensor pointer");
@@ -146,6 +175,7 @@ int hiprwkv_wkv7_step(hiprwkv_stream stream, int io_dtype, int state_dtype, int6
                       void* out, void* new_s, int64_t new_s_batch_stride, unsigned flags) {
   int rc = check_matrix_shape("wkv7_step", io_dtype, state_dtype, B, T, H, N);
   if (rc) return rc;
+  if ((rc = check_flags("wkv7_step", flags)) != HIPRWKV_OK) return rc;
   if (T > HIPRWKV_SMALL_T) return fail(HIPRWKV_EINVAL, "wkv7_step: T=%lld, at most %d tokens per call", (long long)T, HIPRWKV_SMALL_T);
   const void* req[] = {w, r, k, v, a, b, s, out, new_s};
   for (const void* p : req) {
@@ -183,6 +213,7 @@ int hiprwkv_wkv7_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64
                      void* workspace, size_t workspace_bytes, unsigned flags) {
   int rc = check_matrix_shape("wkv7_bwd", io_dtype, state_dtype, B, T, H, N);
   if (rc) return rc;
+  if ((rc = check_flags("wkv7_bwd", flags)) != HIPRWKV_OK) return rc;
   const void* req[] = {w, r, k, v, a, b, s, gy, sa, gw, gr, gk, gv, ga, gb, gs, workspace};
   for (const void* p : req) {
     if (p == nullptr) return fail(HIPRWKV_EINVAL, "wkv7_bwd: null tensor pointer");
@@ -223,6 +254,7 @@ int hiprwkv_wkv6_fwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64
                      const uint32_t* length, const uint8_t* new_starts, void* out, void* new_s, unsigned flags) {
   int rc = check_matrix_shape("wkv6_fwd", io_dtype, state_dtype, B, T, H, N);
   if (rc) return rc;
+  if ((rc = check_flags("wkv6_fwd", flags)) != HIPRWKV_OK) return rc;
   const void* req[] = {r, k, v, w, u, s, out, new_s};
   for (const void* p : req) {
     if (p == nullptr) return fail(HIPRWKV_EINVAL, "wkv6_fwd: null tensor pointer");
@@ -251,6 +283,7 @@ int hiprwkv_wkv6_step(hiprwkv_stream stream, int io_dtype, int state_dtype, int6
                       int64_t new_s_batch_stride, unsigned flags) {
   int rc = check_matrix_shape("wkv6_step", io_dtype, state_dtype, B, T, H, N);
   if (rc) return rc;
+  if ((rc = check_flags("wkv6_step", flags)) != HIPRWKV_OK) return rc;
   if (T > HIPRWKV_SMALL_T) return fail(HIPRWKV_EINVAL, "wkv6_step: T=%lld, at most %d tokens per call", (long long)T, HIPRWKV_SMALL_T);
   const void* req[] = {r, k, v, w, u, s, out, new_s};
   for (const void* p : req) {
@@ -288,6 +321,7 @@ int hiprwkv_wkv6_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64
                      unsigned flags) {
   int rc = check_matrix_shape("wkv6_bwd", io_dtype, state_dtype, B, T, H, N);
   if (rc) return rc;
+  if ((rc = check_flags("wkv6_bwd", flags)) != HIPRWKV_OK) return rc;
   const void* req[] = {r, k, v, w, u, s, gy, gr, gk, gv, gw, gu, gs, workspace};
   for (const void* p : req) {
     if (p == nullptr) return fail(HIPRWKV_EINVAL, "wkv6_bwd: null tensor pointer");
@@ -350,6 +384,7 @@ int hiprwkv_wkv4_fwd_ckpt(hiprwkv_stream stream, int io_dtype, int64_t B, int64_
 static int wkv4_fwd_impl(hiprwkv_stream stream, int io_dtype, int64_t B, int64_t T, int64_t C, const void* w,
                          const void* u, const void* k, const void* v, const void* s, const uint32_t* length,
                          const uint8_t* new_starts, void* new_s, void* out, float* ckpt, unsigned flags) {
+  if (int rc = check_flags("wkv4_fwd", flags)) return rc;
   if (!dtype_ok(io_dtype)) return fail(HIPRWKV_EINVAL, "wkv4_fwd: dtype must be HIPRWKV_F32 or HIPRWKV_BF16");
   if (B <= 0 || T <= 0 || C <= 0) return fail(HIPRWKV_EINVAL, "wkv4_fwd: B,T,C must be positive");
   if (B * ((C + 63) / 64) > 0x7fffffffLL) return fail(HIPRWKV_EINVAL, "wkv4_fwd: B*C exceeds the grid limit");
@@ -382,6 +417,7 @@ int hiprwkv_wkv4_bwd(hiprwkv_stream stream, int io_dtype, int64_t B, int64_t T, 
                      const void* u, const void* k, const void* v, const void* gy, const void* s,
                      const uint32_t* length, const uint8_t* new_starts, const void* gs_new, float* gw, float* gu,
                      void* gk, void* gv, void* gs, void* workspace, size_t workspace_bytes, unsigned flags) {
+  if (int rc = check_flags("wkv4_bwd", flags)) return rc;
   if (!dtype_ok(io_dtype)) return fail(HIPRWKV_EINVAL, "wkv4_bwd: dtype must be HIPRWKV_F32 or HIPRWKV_BF16");
   if (B <= 0 || T <= 0 || C <= 0) return fail(HIPRWKV_EINVAL, "wkv4_bwd: B,T,C must be positive");
   if (B * ((C + 63) / 64) > 0x7fffffffLL) return fail(HIPRWKV_EINVAL, "wkv4_bwd: B*C exceeds the grid limit");
@@ -417,6 +453,9 @@ int hiprwkv_wkv4_bwd_noalloc(hiprwkv_stream stream, int io_dtype, int64_t B, int
                              const uint32_t* length, const uint8_t* new_starts, const void* gs_new, float* gw,
                              float* gu, void* gk, void* gv, void* gs, unsigned flags) {
   if (B <= 0 || T <= 0 || C <= 0) return fail(HIPRWKV_EINVAL, "wkv4_bwd_noalloc: B,T,C must be positive");
+  // the shared scratch array holds whatever the last call left: this entry point always writes its own checkpoints
+  if (flags & HIPRWKV_CKPT_READY)
+    return fail(HIPRWKV_EINVAL, "wkv4_bwd_noalloc: HIPRWKV_CKPT_READY is not accepted (the built-in scratch is shared between calls)");
   const size_t need = hiprwkv_wkv4_bwd_workspace_bytes(B, T, C);
   if (need > SCRATCH_BYTES)
     return fail(HIPRWKV_ENOSPACE,

@@ -189,8 +189,10 @@ __device__ __forceinline__ float row_scan(float x) {
 // E: inclusive running sums (log2 decay, <= 0, non-increasing along the row) of 8 channels over the 16 token lanes.
 // A channel whose total over the chunk is below MIN_CUM_L2 has all its steps of this chunk scaled by the same
 // factor so that the total becomes MIN_CUM_L2: 1/E stays finite in fp32 and the relative weights inside the chunk
-// keep their order, at the price of an inexact (weaker) decay for that channel in that chunk.
-__device__ __forceinline__ void cap_chunk_decay(float (&E)[8], int lane) {
+// keep their order, at the price of an inexact (weaker) decay for that channel in that chunk.  Every wave that caps
+// a channel adds one to the library's numeric-event counter (`events`, may be null), so the inexact result does not
+// pass unnoticed.
+__device__ __forceinline__ void cap_chunk_decay(float (&E)[8], int lane, unsigned* events) {
   // one comparison of the smallest of the eight sums instead of eight
   const float lo = fminf(fminf(fminf(E[0], E[1]), fminf(E[2], E[3])), fminf(fminf(E[4], E[5]), fminf(E[6], E[7])));
   if (__ballot(lo < MIN_CUM_L2) != 0ull) {
@@ -200,7 +202,20 @@ __device__ __forceinline__ void cap_chunk_decay(float (&E)[8], int lane) {
       const float tot = __shfl(E[e], (lane & 48) | 15, 64);
       if (tot < MIN_CUM_L2) E[e] *= MIN_CUM_L2 / tot;
     }
+    if (lane == 0 && events != nullptr) atomicAdd(events, 1u);
   }
+}
+// The numeric-event word sits right behind the hand-shake failure word (api.hip: g_status_words).
+__device__ __forceinline__ unsigned* events_word(unsigned* status) { return status != nullptr ? status + 1 : nullptr; }
+// Non-finite values in a carried 64x64 state (an fp16 operand overflowed: |state|, |sa|, |v| or a scaled input beyond
+// 65504): one numeric event per wave that sees one.  Called once per consumer wave, after the last chunk.
+__device__ __forceinline__ void count_nonfinite(const f32x4_t (&S)[4], int lane, unsigned* events) {
+  float z = 0.f;
+#pragma unroll
+  for (int tile = 0; tile < 4; ++tile)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) z = fmaf(S[tile][i], 0.f, z);      // 0 for finite values, NaN for an inf or a NaN
+  if (__ballot(!(z == 0.f)) != 0ull && lane == 0 && events != nullptr) atomicAdd(events, 1u);
 }
 
 // value of the previous lane of the row; `first` in lane 0 of the row

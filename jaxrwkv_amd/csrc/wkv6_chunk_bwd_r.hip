@@ -92,7 +92,7 @@ struct Producer {
 };
 
 __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const ChunkFlags& F, Slot* __restrict__ slot,
-                                        SnapSlot* __restrict__ snap) {
+                                        SnapSlot* __restrict__ snap, unsigned* events) {
   const int lane = P.lane, t = lane & 15, g = lane >> 4;
   const bool valid = t < F.nvalid;
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -145,7 +145,7 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
           if (F.nvalid != CK) l2 = valid ? l2 : 0.f;
           E[e] = row_scan(l2);
         }
-        cap_chunk_decay(E, lane);
+        cap_chunk_decay(E, lane, events);
       }
       if (slow) {
 #pragma unroll
@@ -647,7 +647,7 @@ __global__ __launch_bounds__(64 * (NCONS_R + NPROD)) void wkv6_chunk_bwd_r_kerne
       const int si = j % RING;
       Slot* slot = &slots[si];
       if (j >= RING && !wait_consumed(sy, si, j - RING + 1, lane)) break;
-      produce(P, raw, F, slot, snapslot);
+      produce(P, raw, F, slot, snapslot, events_word(A.status));
       if (j + NPROD < nch) load_raw(raw, A, b, h, (int64_t)(c - NPROD) * CK, lane);
       if ((A.flags & FLAG_DROP_PUBLISH) && j + 1 == nch) break;
       if (lane == 0) __hip_atomic_store(&sy->ready[si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);

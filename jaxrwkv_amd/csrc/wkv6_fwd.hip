@@ -129,7 +129,7 @@ __device__ __forceinline__ void mask_raw(Raw& x, int nvalid, int lane) {
 
 // Everything of one chunk that does not depend on the carried state.  `ulds`: the bonus u of this head in LDS (bf16).
 __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags& F, const uint16_t* __restrict__ ulds,
-                                        Slot* __restrict__ slot, SnapSlot* __restrict__ snap) {
+                                        Slot* __restrict__ slot, SnapSlot* __restrict__ snap, unsigned* events) {
   const int t = lane & 15, g = lane >> 4;
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
   const uint4 zero16 = make_uint4(0u, 0u, 0u, 0u);
@@ -177,7 +177,7 @@ __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags
       }
 #pragma unroll
       for (int e = 0; e < 8; ++e) E[e] = row_scan(fw[e]);
-      cap_chunk_decay(E, lane);
+      cap_chunk_decay(E, lane, events);
     }
     if (slow) {
       rare_path();
@@ -493,6 +493,8 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv6_fwd_kernel(Wkv6Args
       // every LDS read of slot si has returned: its data went into the MFMAs above
       if (lane == 0) __hip_atomic_store(&sy->consumed[cq][si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
+    // an operand beyond the fp16 range leaves inf or NaN in the carried state (until a reset discards it): count it
+    count_nonfinite(C.S, lane, events_word(A.status));
   } else {
     const int p = wave - NCONS;
     Raw raw;
@@ -503,7 +505,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv6_fwd_kernel(Wkv6Args
       const int si = j % RING;
       if (j >= RING && !wait_consumed_lazy(sy, si, j - RING + 1, lane)) break;
       mask_raw(raw, F.nvalid, lane);
-      produce(lane, raw, F, ulds, &slots[si], snapslot);
+      produce(lane, raw, F, ulds, &slots[si], snapslot, events_word(A.status));
       if (j + NPROD < nch) load_raw(raw, A, b, h, c0 + (int64_t)NPROD * CK, lane);
       if ((A.flags & FLAG_DROP_PUBLISH) && j + 1 == nch) break;
       // the release orders this wave's LDS writes before the sequence number

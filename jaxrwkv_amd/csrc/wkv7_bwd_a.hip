@@ -113,7 +113,7 @@ struct Producer {
 // same pipeline one after the other (scan, scaling, hi/lo split, LDS parking, transposes, partial Gram sums),
 // which keeps the live register set small.
 __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const ChunkFlags& F, Slot* __restrict__ slot,
-                                        SnapSlot* __restrict__ snap) {
+                                        SnapSlot* __restrict__ snap, unsigned* events) {
   const int lane = P.lane, t = lane & 15, g = lane >> 4;
   const bool valid = t < F.nvalid;
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -180,7 +180,7 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
       }
 #pragma unroll
       for (int e = 0; e < 8; ++e) E[e] = row_scan(fw[e]);
-      cap_chunk_decay(E, lane);
+      cap_chunk_decay(E, lane, events);
     }
     unpack8(x.a[hf], fa);
     if (slow) {
@@ -635,7 +635,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_bwd_a_kernel(Wkv7Ar
       Slot* slot = &slots[si];
       if (j >= RING && !wait_consumed(sy, si, j - RING + 1, lane)) break;
       mask_raw(raw, F.nvalid, lane);
-      produce(P, raw, F, slot, snapslot);
+      produce(P, raw, F, slot, snapslot, events_word(A.status));
       if (j + NPROD < nch) load_raw(raw, A, b, h, (int64_t)(c - NPROD) * CK, lane);
       if ((A.flags & FLAG_DROP_PUBLISH) && j + 1 == nch) break;
       // the release orders this wave's LDS writes before the sequence number

@@ -119,7 +119,7 @@ __device__ __forceinline__ void split8h(const uint4 raw, u32x4_t& h, u32x4_t& l)
 }
 
 __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const ChunkFlags& F, Slot* __restrict__ slot,
-                                        SnapSlot* __restrict__ snap) {
+                                        SnapSlot* __restrict__ snap, unsigned* events) {
   const int lane = P.lane, t = lane & 15, g = lane >> 4;
   const bool valid = t < F.nvalid;
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -173,7 +173,7 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
           if (F.nvalid != CK) l2 = valid ? l2 : 0.f;
           E[e] = row_scan(l2);
         }
-        cap_chunk_decay(E, lane);
+        cap_chunk_decay(E, lane, events);
       }
       if (slow) {
 #pragma unroll
@@ -586,7 +586,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_bwd_c_kernel(
       const int si = j % RING;
       Slot* slot = &slots[si];
       if (j >= RING && !wait_consumed(sy, si, j - RING + 1, lane)) break;
-      produce(P, raw, F, slot, snapslot);
+      produce(P, raw, F, slot, snapslot, events_word(A.status));
       if (j + NPROD < nch) load_raw(raw, A, b, h, (int64_t)(c - NPROD) * CK, lane);
       if ((A.flags & FLAG_DROP_PUBLISH) && j + 1 == nch) break;
       // the release orders this wave's LDS writes before the sequence number

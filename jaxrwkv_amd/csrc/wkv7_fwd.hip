@@ -139,7 +139,7 @@ __device__ __forceinline__ uint4 pack_h8(const float (&f)[8]) {
 // Everything of one chunk that does not depend on the carried state.  The two 32-key halves go through the same
 // pipeline one after the other, which keeps the live register set small.
 __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags& F, Slot* __restrict__ slot,
-                                        SnapSlot* __restrict__ snap) {
+                                        SnapSlot* __restrict__ snap, unsigned* events) {
   const int t = lane & 15, g = lane >> 4;
   const bool valid = t < F.nvalid;
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -194,7 +194,7 @@ __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags
       }
 #pragma unroll
       for (int e = 0; e < 8; ++e) E[e] = row_scan(fw[e]);
-      cap_chunk_decay(E, lane);
+      cap_chunk_decay(E, lane, events);
     }
     unpack8(x.a[hf], fa);
     if (slow) {
@@ -613,6 +613,8 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_fwd_kernel(Wkv7Args
       // every LDS read of slot si has returned: its data went into the MFMAs above
       if (lane == 0) __hip_atomic_store(&sy->consumed[cq][si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
+    // an operand beyond the fp16 range leaves inf or NaN in the carried state (until a reset discards it): count it
+    count_nonfinite(C.S, lane, events_word(A.status));
   } else {
     const int p = pp;
     Raw raw;
@@ -624,7 +626,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_fwd_kernel(Wkv7Args
       Slot* slot = &slots[si];
       if (j >= RING && !wait_consumed_lazy(sy, si, j - RING + 1, lane)) break;
       mask_raw(raw, F.nvalid, lane);
-      produce(lane, raw, F, slot, snapslot);
+      produce(lane, raw, F, slot, snapslot, events_word(A.status));
       if (j + NPROD < nch) load_raw(raw, A, b, h, c0 + (int64_t)NPROD * CK, lane);
       if ((A.flags & FLAG_DROP_PUBLISH) && j + 1 == nch) break;
       // the release orders this wave's LDS writes before the sequence number

@@ -111,7 +111,7 @@ __device__ __forceinline__ void put2(float* row, int hf, int g, const float (&f)
 // Everything of one chunk that does not depend on the carried state.  The two 32-key halves (j = 0,1 and j = 2,3) go
 // through the same pipeline one after the other, which keeps the live register set small.
 __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags& F, Slot* __restrict__ slot,
-                                        SnapSlot* __restrict__ snap, TrTile* __restrict__ tr) {
+                                        SnapSlot* __restrict__ snap, TrTile* __restrict__ tr, unsigned* events) {
   const int t = lane & 15, g = lane >> 4;
   const bool valid = t < F.nvalid;
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -177,7 +177,7 @@ __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags
           E[e] += El[e];
           El[e] = 0.f;
         }
-        cap_chunk_decay(E, lane);
+        cap_chunk_decay(E, lane, events);
       }
     }
     unpack2(x.a[2 * hf], x.a[2 * hf + 1], fa);
@@ -580,7 +580,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_fwd_f32_kernel(Wkv7
       const int si = j % RING;
       if (j >= RING && !wait_consumed_lazy(sy, si, j - RING + 1, lane)) break;
       mask_raw(raw, F.nvalid, lane);
-      produce(lane, raw, F, &slots[si], snapslot, &trs[p]);
+      produce(lane, raw, F, &slots[si], snapslot, &trs[p], events_word(A.status));
       if (j + NPROD < nch) load_raw(raw, A, b, h, c0 + (int64_t)NPROD * CK, lane);
       if ((A.flags & FLAG_DROP_PUBLISH) && j + 1 == nch) break;
       // the release orders this wave's LDS writes before the sequence number

@@ -12,8 +12,9 @@ support and ``libhiprwkv_xla.so`` (``python -m jaxrwkv_amd.build --xla-ffi``, ha
 
 Differences from the reference's ``wkv7_cuda`` (rwkv7.py:356-446): no ``s_restore`` residual and no ``T % 16`` /
 ``T == 1`` special cases; gradients reach ``s`` and come from the returned state; ``new_starts`` is honoured in the
-backward pass; batching is ``vmap_method="broadcast_all"`` (every leading axis is one flat batch inside the
-handler), so no ``custom_vmap`` rules are needed.  Results equal ``AssociativeScanRWKV`` (``COMPAT_ASSOC``).
+backward pass; every leading axis is one flat batch inside the handler, and a ``custom_vmap`` rule (``_call``) keeps
+the per-model parameters (WKV6 ``u``, WKV4 ``w`` and ``u``) un-batched and refuses a vmap over them.  Results equal
+``AssociativeScanRWKV`` (``COMPAT_ASSOC``).
 """
 import ctypes
 import os
@@ -47,17 +48,38 @@ def register():
     _registered = True
 
 
-def _call(target, result_types, *operands):
-    # vmap_method="broadcast_all" hands a vmapped call to the handler with the mapped axes as extra LEADING
-    # dimensions on every operand (unmapped operands are broadcast to the same leading shape, at the cost of a
-    # copy).  The handlers in csrc/xla_ffi.cc rely on exactly that: they take the last three (WKV4: two) dimensions
-    # as (T, H, N) and fold everything before them into one flat batch B, for the state, length and new_starts
-    # operands too.  An operand vmapped with a non-leading out-axis would break this; jax.ffi never produces one.
-    # The per-head / per-channel parameters (WKV6 u (H,N), WKV4 w and u (C,)) then arrive with the same leading batch
-    # shape, and the C ABI reads only the first (H,N) / (C,) of them: right when they were broadcast, which is the
-    # reference's use (one parameter set per model), and silently wrong for a caller that vmaps over per-example
-    # parameters.
-    return jax.ffi.ffi_call(target, result_types, vmap_method="broadcast_all")(*operands, flags=np.int64(COMPAT_ASSOC))
+def _call(target, result_types, *operands, params=()):
+    """One XLA custom call.  ``params`` lists the positions of per-model parameters among the operands (WKV6 ``u``
+    (H,N), WKV4 ``w`` and ``u`` (C,)): the C ABI takes exactly one set of them per call.
+
+    Batching.  The handlers in csrc/xla_ffi.cc take the last three (WKV4: two) dimensions of the token operands as
+    (T, H, N) and fold everything before them into one flat batch, for the state, length and new_starts operands too;
+    the parameters must arrive at their own rank.  A plain ``vmap_method="broadcast_all"`` would hand a vmapped call
+    the parameters broadcast to the batch shape (or, for a caller that maps over per-example parameters, B different
+    sets of which only the first would be read).  The call is therefore wrapped in a ``custom_vmap`` rule that keeps
+    the parameters un-batched, broadcasts every other un-mapped operand to the mapped axis (at the cost of a copy,
+    as ``broadcast_all`` does), and raises for a vmap over a parameter.  The rule calls the wrapped function again, so
+    nested vmaps add one leading axis each."""
+    params = tuple(params)
+
+    @jax.custom_batching.custom_vmap
+    def call(*ops):
+        return tuple(jax.ffi.ffi_call(target, result_types(*ops), vmap_method="broadcast_all")(
+            *ops, flags=np.int64(COMPAT_ASSOC)))
+
+    @call.def_vmap
+    def _rule(axis_size, in_batched, *ops):
+        for i in params:
+            if in_batched[i]:
+                raise NotImplementedError(
+                    f"{target}: operand {i} is a per-model parameter; the kernel takes one set per call, so a vmap "
+                    "over it (per-example parameters) is not supported -- loop over the parameter sets instead")
+        ops = tuple(x if (bt or i in params) else jnp.broadcast_to(x[None], (axis_size,) + jnp.shape(x))
+                    for i, (x, bt) in enumerate(zip(ops, in_batched)))
+        outs = call(*ops)
+        return outs, tuple(True for _ in outs)
+
+    return call(*operands)
 
 
 def _sds(x, dtype=None):
@@ -78,19 +100,22 @@ def wkv7_hip(r, w, k, v, a, b, s, length, new_starts):
 def _wkv7_fwd(r, w, k, v, a, b, s, length, new_starts):
     register()
     length = jnp.uint32(length)
-    out, sa, new_s = _call("hip-wkv7-fwd", (_sds(r), _sds(r, jnp.float32 if r.dtype == jnp.float32 else jnp.float16), _sds(s)),
-                           w, r, k, v, a, b, s, length, new_starts)
+    # the residual sa is fp32 beside fp32 I/O and IEEE half beside bf16 I/O (the reference's sa_restore is fp32 for
+    # both, rwkv7.py:364); the handlers check the element type against r's
+    types = lambda w, r, k, v, a, b, s, length, new_starts: (
+        _sds(r), _sds(r, jnp.float32 if r.dtype == jnp.float32 else jnp.float16), _sds(s))
+    out, sa, new_s = _call("hip-wkv7-fwd", types, w, r, k, v, a, b, s, length, new_starts)
     return (new_s, out), (r, w, k, v, a, b, s, length, new_starts, sa)
 
 
 def _wkv7_bwd(res, grads):
     r, w, k, v, a, b, s, length, new_starts, sa = res
     gs_out, gy = grads
-    T, H, N = r.shape[-3:]
-    nbytes = register.lib.hiprwkv_wkv7_bwd_workspace_bytes(int(np.prod(r.shape[:-3], dtype=np.int64)), T, H, N)
-    ws = jax.ShapeDtypeStruct((nbytes,), jnp.uint8)
-    gw, gr, gk, gv, ga, gb, gs, _ = _call("hip-wkv7-bwd", tuple(_sds(x) for x in (w, r, k, v, a, b, s)) + (ws,),
-                                          w, r, k, v, a, b, s, length, new_starts, gy, sa, gs_out)
+    def types(w, r, k, v, a, b, s, length, new_starts, gy, sa, gs_out):
+        T, H, N = r.shape[-3:]
+        nbytes = register.lib.hiprwkv_wkv7_bwd_workspace_bytes(int(np.prod(r.shape[:-3], dtype=np.int64)), T, H, N)
+        return tuple(_sds(x) for x in (w, r, k, v, a, b, s)) + (jax.ShapeDtypeStruct((nbytes,), jnp.uint8),)
+    gw, gr, gk, gv, ga, gb, gs, _ = _call("hip-wkv7-bwd", types, w, r, k, v, a, b, s, length, new_starts, gy, sa, gs_out)
     return (gr, gw, gk, gv, ga, gb, gs) + _zero_cotangents(length, new_starts)
 
 
@@ -112,20 +137,24 @@ def wkv6_hip(r, k, v, w, u, s, length, new_starts):
 def _wkv6_fwd(r, k, v, w, u, s, length, new_starts):
     register()
     length = jnp.uint32(length)
-    out, new_s = _call("hip-wkv6-fwd", (_sds(r), _sds(s)), r, k, v, w, u, s, length, new_starts)
+    types = lambda r, k, v, w, u, s, length, new_starts: (_sds(r), _sds(s))
+    out, new_s = _call("hip-wkv6-fwd", types, r, k, v, w, u, s, length, new_starts, params=(4,))
     return (new_s, out), (r, k, v, w, u, s, length, new_starts)
 
 
 def _wkv6_bwd(res, grads):
     r, k, v, w, u, s, length, new_starts = res
     gs_out, gy = grads
-    T, H, N = r.shape[-3:]
-    lead = r.shape[:-3]
-    nbytes = register.lib.hiprwkv_wkv6_bwd_workspace_bytes(int(np.prod(lead, dtype=np.int64)), T, H, N)
-    gu_t = jax.ShapeDtypeStruct(lead + (H, N), jnp.float32)
-    gr, gk, gv, gw, gu, gs, _ = _call("hip-wkv6-bwd", (_sds(r), _sds(k), _sds(v), _sds(w), gu_t, _sds(s),
-                                                       jax.ShapeDtypeStruct((nbytes,), jnp.uint8)),
-                                      r, k, v, w, u, s, length, new_starts, gy, gs_out)
+    H, N = r.shape[-2:]
+
+    def types(r, k, v, w, u, s, length, new_starts, gy, gs_out):
+        T, H, N = r.shape[-3:]
+        lead = r.shape[:-3]
+        nbytes = register.lib.hiprwkv_wkv6_bwd_workspace_bytes(int(np.prod(lead, dtype=np.int64)), T, H, N)
+        return (_sds(r), _sds(k), _sds(v), _sds(w), jax.ShapeDtypeStruct(lead + (H, N), jnp.float32), _sds(s),
+                jax.ShapeDtypeStruct((nbytes,), jnp.uint8))
+    gr, gk, gv, gw, gu, gs, _ = _call("hip-wkv6-bwd", types, r, k, v, w, u, s, length, new_starts, gy, gs_out,
+                                      params=(4,))
     gu = gu.reshape((-1, H, N)).sum(0).astype(u.dtype).reshape(u.shape)
     return (gr, gk, gv, gw, gu, gs) + _zero_cotangents(length, new_starts)
 
@@ -148,20 +177,24 @@ def wkv4_hip(w_neg, u, k, v, s, length, new_starts):
 def _wkv4_fwd(w_neg, u, k, v, s, length, new_starts):
     register()
     length = jnp.uint32(length)
-    new_s, out = _call("hip-wkv4-fwd", (_sds(s), _sds(k)), w_neg, u, k, v, s, length, new_starts)
+    types = lambda w_neg, u, k, v, s, length, new_starts: (_sds(s), _sds(k))
+    new_s, out = _call("hip-wkv4-fwd", types, w_neg, u, k, v, s, length, new_starts, params=(0, 1))
     return (new_s, out), (w_neg, u, k, v, s, length, new_starts)
 
 
 def _wkv4_bwd(res, grads):
     w_neg, u, k, v, s, length, new_starts = res
     gs_new, gy = grads
-    T, C = k.shape[-2:]
-    lead = k.shape[:-2]
-    nbytes = register.lib.hiprwkv_wkv4_bwd_workspace_bytes(int(np.prod(lead, dtype=np.int64)), T, C)
-    per_seq = jax.ShapeDtypeStruct(lead + (C,), jnp.float32)
-    gw, gu, gk, gv, gs, _ = _call("hip-wkv4-bwd", (per_seq, per_seq, _sds(k), _sds(v), _sds(s),
-                                                   jax.ShapeDtypeStruct((nbytes,), jnp.uint8)),
-                                  w_neg, u, k, v, gy, s, length, new_starts, gs_new)
+    C = k.shape[-1]
+
+    def types(w_neg, u, k, v, gy, s, length, new_starts, gs_new):
+        T, C = k.shape[-2:]
+        lead = k.shape[:-2]
+        nbytes = register.lib.hiprwkv_wkv4_bwd_workspace_bytes(int(np.prod(lead, dtype=np.int64)), T, C)
+        per_seq = jax.ShapeDtypeStruct(lead + (C,), jnp.float32)
+        return (per_seq, per_seq, _sds(k), _sds(v), _sds(s), jax.ShapeDtypeStruct((nbytes,), jnp.uint8))
+    gw, gu, gk, gv, gs, _ = _call("hip-wkv4-bwd", types, w_neg, u, k, v, gy, s, length, new_starts, gs_new,
+                                  params=(0, 1))
     gw = gw.reshape((-1, C)).sum(0).astype(w_neg.dtype)          # summed over the batch as in rwkv4.py:351
     gu = gu.reshape((-1, C)).sum(0).astype(u.dtype)
     return (gw, gu, gk, gv, gs) + _zero_cotangents(length, new_starts)

@@ -62,6 +62,17 @@ def handshake_failures():
     return int(n.value)
 
 
+def numeric_events():
+    """Numeric events of the chunked kernels since the library was loaded: waves that capped a channel's decay over a
+    chunk at e^-80 (its result is then inexact) and waves that found inf or NaN in a carried state of the bf16
+    forward kernels (an IEEE-half operand overflowed: |state|, |sa|, |v| beyond 65504).  Synchronises the current
+    stream."""
+    lib = _lib.load()
+    n = ctypes.c_uint(0)
+    _lib.check(lib.hiprwkv_numeric_events(_stream(), ctypes.byref(n)), "hiprwkv_numeric_events")
+    return int(n.value)
+
+
 # ----------------------------------------------------------------------------- WKV7
 def wkv7_fwd(r, w, k, v, a, b, s, length=None, new_starts=None, compat=True, want_sa=False, force_seq=False,
              small_t=True, debug_flags=0):

@@ -153,3 +153,51 @@ def test_xla_ffi_sources_agree_on_symbols_and_abi():
     assert defined == registered and len(defined) == 6
     for fn in set(re.findall(r"\b(hiprwkv_\w+)\(", cc)):
         assert re.search(r"\b%s\(" % fn, header), fn
+    # Each handler's parameter list and its binding declare the same number of buffers, in the same kinds.
+    for name in defined:
+        fn = name.replace("Hip", "")
+        params = re.search(r"ffi::Error %s\(hipStream_t stream,(.*?)\) \{" % fn, cc, re.S).group(1)
+        bind = re.search(r"XLA_FFI_DEFINE_HANDLER_SYMBOL\(%s, %s,(.*?)\);" % (name, fn), cc, re.S).group(1)
+        p_args = re.findall(r"ffi::(AnyBuffer|Buffer<ffi::\w+>) \w+", re.sub(r"ffi::Result<ffi::(?:AnyBuffer|Buffer<ffi::\w+>)> \w+", "", params))
+        p_rets = re.findall(r"ffi::Result<ffi::(AnyBuffer|Buffer<ffi::\w+>)> \w+", params)
+        b_args = re.findall(r"\.Arg<ffi::(AnyBuffer|Buffer<ffi::\w+>)>\(\)", bind)
+        b_rets = re.findall(r"\.Ret<ffi::(AnyBuffer|Buffer<ffi::\w+>)>\(\)", bind)
+        assert p_args == b_args, (name, p_args, b_args)
+        assert p_rets == b_rets, (name, p_rets, b_rets)
+    # The WKV7 residual is half beside bf16 I/O: both handlers check its element type against r's, the token operands
+    # against each other, and the binding declares the matching result type.
+    assert cc.count("sa_type_ok(r.element_type()") == 2 and "io == ffi::BF16 && sa == ffi::F16" in cc
+    assert "jnp.float32 if r.dtype == jnp.float32 else jnp.float16" in py
+    # Per-model parameters must arrive un-batched: rank checks in the handlers, a custom_vmap rule in the binding.
+    assert cc.count("one parameter set per call") >= 4
+    assert "custom_vmap" in py and "params=(4,)" in py and "params=(0, 1)" in py
+    # The debug hook cannot come in through the XLA attribute.
+    assert "static_cast<unsigned>(flags) & HIPRWKV_PUBLIC_FLAGS" in cc and cc.count("public_flags(flags)") == 6
+
+
+def test_flag_bits_are_validated_without_gpu():
+    """Unknown flag bits are refused; the debug hook is refused unless the process environment enables it (checked in
+    a child process, because the library reads the variable once); the entry point that allocates nothing refuses
+    HIPRWKV_CKPT_READY (its scratch array is shared between calls)."""
+    import subprocess
+    import sys
+    from jaxrwkv_amd import _lib
+    lib = _lib.load()
+    null = ctypes.c_void_p(0)
+    rc = lib.hiprwkv_wkv7_fwd(null, 0, 0, 1, 8, 1, 64, *([null] * 12), 0x4000)
+    assert rc == -1 and b"unknown flag" in lib.hiprwkv_last_error()
+    rc = lib.hiprwkv_wkv4_fwd(null, 0, 1, 8, 64, *([null] * 9), 0x8)
+    assert rc == -1 and b"unknown flag" in lib.hiprwkv_last_error()
+    ok = ctypes.c_void_p(0x10000)
+    rc = lib.hiprwkv_wkv4_bwd_noalloc(null, 0, 1, 8, 64, *([ok] * 6), null, null, null, *([ok] * 5), _lib.CKPT_READY)
+    assert rc == -1 and b"CKPT_READY" in lib.hiprwkv_last_error()
+    code = ("import ctypes; from jaxrwkv_amd import _lib; lib = _lib.load(); n = ctypes.c_void_p(0); "
+            "rc = lib.hiprwkv_wkv7_fwd(n, 0, 0, 1, 8, 1, 64, *([n] * 12), 0x100); "
+            "print(rc, lib.hiprwkv_last_error().decode())")
+    for enable, want in ((None, "HIPRWKV_ENABLE_DEBUG_FLAGS"), ("1", "null tensor pointer")):
+        env = {k: v for k, v in os.environ.items() if k != "HIPRWKV_ENABLE_DEBUG_FLAGS"}
+        if enable:
+            env["HIPRWKV_ENABLE_DEBUG_FLAGS"] = enable
+        out = subprocess.run([sys.executable, "-c", code], cwd=ROOT, env=env, capture_output=True, text=True, timeout=120)
+        assert out.returncode == 0, out.stderr
+        assert out.stdout.startswith("-1 ") and want in out.stdout, out.stdout

@@ -1,8 +1,13 @@
 """The chunked kernels' bounded hand-shake fails loudly: with HIPRWKV_DEBUG_DROP_PUBLISH the producer of the last
 chunk never publishes it, the consumers' wait runs out, every wave still ends normally (the launch returns, later
 launches work), all outputs of every (sequence, head) are NaN and the failure counter advances by B*H per kernel."""
+import os
+
 import pytest
 import torch
+
+# the library accepts the test hook only in a process that asks for it (read at the first call that carries the flag)
+os.environ["HIPRWKV_ENABLE_DEBUG_FLAGS"] = "1"
 
 pytestmark = pytest.mark.gpu
 

@@ -99,28 +99,58 @@ def test_matches_sequential_kernel_and_tvd_bar():
     assert tvd_unrounded.max() < tvd_floor.max() + 5e-4, (tvd_unrounded.max(), tvd_floor.max())
 
 
-def test_strong_decay_is_finite():
-    # decays far below the clamp must not produce inf/nan; with w <= 1.6 the result still matches the oracle
+def test_strong_decay_is_finite_and_counted():
+    """A key channel whose log decay over a 16-token chunk is below -80 gets that chunk's steps scaled to -80 in
+    total: finite, inexact, and counted by hiprwkv_numeric_events.  Decays above the floor are exact and silent."""
+    from jaxrwkv_amd import ops
     x = wkv7_inputs(1, 64, 1, 64, seed=51, bf16=True, resets=False, lengths=False)
-    x["w"] = bf16_round(np.clip(x["w"] + 1.5, None, 1.6)).astype(np.float64)
+    x["w"] = bf16_round(np.clip(x["w"] + 1.5, None, 1.6)).astype(np.float64)    # exp(1.6) * 16 = 79.2 < 80
+    before = ops.numeric_events()
     new_s, y, sa = run(x, False)
     check(x, False, new_s, y, sa)
-    x["w"][:] = 4.0
+    assert ops.numeric_events() == before                  # no chunk reached the floor
+    x["w"][:] = 4.0                                         # exp(4) * 16 = 874: every chunk of every channel
     new_s, y, sa = run(x, False)
     assert np.all(np.isfinite(y)) and np.all(np.isfinite(new_s))
+    assert ops.numeric_events() >= before + 4 * 2           # four chunks, two 32-key halves each
+    # the fp32-I/O chunked kernel has the same floor and counts the same way
+    before = ops.numeric_events()
+    t = {n: dev(x[n]) for n in "rwkvab"}
+    s32, y32, _ = ops.wkv7_fwd(t["r"], t["w"], t["k"], t["v"], t["a"], t["b"], dev(x["s"]), small_t=False)
+    assert bool(torch.isfinite(y32).all()) and ops.numeric_events() >= before + 4 * 2
+    # the sequential kernels have no floor: nothing is counted there
+    before = ops.numeric_events()
+    ops.wkv7_fwd(t["r"], t["w"], t["k"], t["v"], t["a"], t["b"], dev(x["s"]), small_t=False, force_seq=True)
+    assert ops.numeric_events() == before
 
 
-def test_values_beyond_the_fp16_range_are_loud_not_wrong():
-    """The bf16 forward feeds fp16 operands to the matrix cores: v (and with it the state) beyond 65504 cannot be
-    represented.  The conversion overflows to infinity, so y comes back non-finite instead of plausible-but-wrong;
-    the sequential kernel (HIPRWKV_FORCE_SEQ) has no such limit and still matches the oracle."""
+def test_values_beyond_the_fp16_range_give_inf_and_are_counted():
+    """The bf16 forward feeds IEEE-half operands to the matrix cores: v (and with it the state) beyond 65504 cannot
+    be represented.  The conversion overflows to infinity, so y and the state come back non-finite from that token
+    on, and hiprwkv_numeric_events advances; the sequential kernel (HIPRWKV_FORCE_SEQ) has no such limit and still
+    matches the oracle."""
     from jaxrwkv_amd import ops
     x = wkv7_inputs(1, 64, 1, 64, seed=77, bf16=True, resets=False, lengths=False)
     x["v"] = bf16_round(x["v"] * 1.0e5).astype(np.float64)
     t = {n: dev(x[n], torch.bfloat16) for n in "rwkvab"}
+    before = ops.numeric_events()
     _, y, _ = ops.wkv7_fwd(t["r"], t["w"], t["k"], t["v"], t["a"], t["b"], dev(x["s"]), small_t=False)
     assert not bool(torch.isfinite(y.float()).all())
+    assert ops.numeric_events() > before
+    before = ops.numeric_events()
     new_s, y, _ = ops.wkv7_fwd(t["r"], t["w"], t["k"], t["v"], t["a"], t["b"], dev(x["s"]), small_t=False, force_seq=True)
+    assert ops.numeric_events() == before
     ref_s, ref_y = o7.wkv7_base(*[x[n] for n in "rwkvab"], x["s"], x["length"], x["new_starts"], compat=True)
     assert_close("y", host(y), ref_y, rtol=2.0 ** -7, atol=1e-4, scale_atol=True)
     assert_close("new_s", host(new_s), ref_s, rtol=1e-4, atol=1e-4, scale_atol=True)
+
+
+@pytest.mark.parametrize("scale", [1.0e-3, 64.0])
+def test_magnitudes_inside_the_documented_range_keep_the_tolerances(scale):
+    """v and the state scaled by 1e-3 or 64: the IEEE-half operands still hold 11 significant bits there, and y, the
+    state and sa stay within the tolerances of the unscaled case (the op is linear in (v, s))."""
+    x = wkv7_inputs(2, 150, 2, 64, seed=83, bf16=True, p_reset=0.02)
+    x["v"] = bf16_round(x["v"] * scale).astype(np.float64)
+    x["s"] = (x["s"] * scale).astype(np.float32).astype(np.float64)
+    new_s, y, sa = run(x, True)
+    check(x, True, new_s, y, sa)

@@ -39,6 +39,28 @@ def test_chosen_formats_meet_the_bf16_bar(case):
     assert m["y"] < 5e-4 and m["s"] < 5e-4 and m["sa"] < 7e-4, m
 
 
+@pytest.mark.parametrize("regime", ["bench", "slow"])
+def test_chosen_formats_meet_the_bar_on_every_seed(regime):
+    """The 1e-3 bar over six more seeds per regime (B=1, T=256, H=2; the slow regime's seed 3 is the worst case found:
+    9.7e-4).  The maximum over positions is dominated by single flips of the bf16 output rounding -- the oracle's own
+    y rounded to bf16 is 4-6e-4 away from the unrounded one by the same measure -- so the mean is pinned as well: it
+    is what the operand formats move (1.3e-4 on benchmark decays, 3.2e-4 on slow ones)."""
+    import numpy as np
+    from .gpu_util import tvd_of_projected
+    from .inputs import bf16_round
+    worst, means = 0.0, []
+    for seed in range(1, 7):
+        x = pm.make_inputs(regime, B=1, T=256, H=2, seed=seed)
+        m, ref = pm.metrics(x, pm.CHOSEN)
+        assert m["tvd_max"] < 1e-3, (regime, seed, m)
+        floor = tvd_of_projected(bf16_round(ref[1]).astype(np.float64), ref[1]).max()
+        assert floor > 3e-4, floor                       # the output format alone costs a third of the bar or more
+        worst = max(worst, m["tvd_max"])
+        means.append(m["tvd_mean"])
+    assert max(means) < (2e-4 if regime == "bench" else 4e-4), means
+    assert worst < 1e-3
+
+
 @pytest.mark.parametrize("name,override", [
     ("single bf16 everywhere", pm.ALL_BF16),
     ("Gram operands single bf16", {**pm.CHOSEN, "gk": "b1", "ga": "b1"}),
