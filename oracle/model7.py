@@ -59,7 +59,14 @@ def channel_mixing_seq(x, state, ffn, length, new_starts):                # rwkv
     return k @ ffn["value"]["weight"].T, x[length - 1]
 
 
-def time_mixing_seq(x, state, v_first, att, length, new_starts, H, S, layer_id):   # rwkv7.py:223-267
+def _bf16(x):
+    """Round to the nearest bfloat16 (ties to even), as float64: the op's I/O format in a bf16 model."""
+    u = np.ascontiguousarray(x, np.float32).view(np.uint32).astype(np.uint64)
+    u = ((u + 0x7FFF + ((u >> 16) & 1)) >> 16) << 16
+    return u.astype(np.uint32).view(np.float32).astype(np.float64)
+
+
+def time_mixing_seq(x, state, v_first, att, length, new_starts, H, S, layer_id, op_io=None):   # rwkv7.py:223-267
     T, C = x.shape
     sx = np.concatenate([state[:1], x[:-1]])
     sx = np.where(new_starts[:, None], 0.0, sx)
@@ -83,17 +90,23 @@ def time_mixing_seq(x, state, v_first, att, length, new_starts, H, S, layer_id):
     state[0] = x[length - 1]
     s = state[1:].reshape(H, S, S)
     r_, w_, k_, v_, a_, b_ = (val.reshape(T, H, S) for val in (r, w, k, v, -kk, kk * a))
-    s_new, out = o7.wkv7_base(r_[None], w_[None], k_[None], v_[None], a_[None], b_[None], s[None],
-                              np.array([length]), new_starts[None], compat=True)
+    op_in = (r_, w_, k_, v_, a_, b_)
+    if op_io == "bf16":      # an op with bf16 I/O: its six inputs and its output are bf16, the state stays wider
+        op_in = tuple(_bf16(val) for val in op_in)
+    s_new, out = o7.wkv7_base(*(val[None] for val in op_in), s[None], np.array([length]), new_starts[None], compat=True)
     state[1:] = s_new[0].reshape(S, -1)
+    if op_io == "bf16":
+        out = _bf16(out)
     y = group_norm_tokens(out[0].reshape(T, H * S), H, att["ln_x"]["weight"], att["ln_x"]["bias"], 64e-5)
     y = y + ((r_ * k_ * att["r_k"]).sum(-1, keepdims=True) * v_).reshape(T, C)
     y = y * g
     return y @ att["output"]["weight"].T, state, v_first
 
 
-def forward(params, tokens, state, length=None, new_starts=None):         # llm.py:71-84, rwkv7.py:269-291
-    """One stream: tokens (T,), state (L, 2+N, C).  Returns (logits (T, vocab), new state)."""
+def forward(params, tokens, state, length=None, new_starts=None, op_io=None):   # llm.py:71-84, rwkv7.py:269-291
+    """One stream: tokens (T,), state (L, 2+N, C).  Returns (logits (T, vocab), new state).  ``op_io="bf16"`` rounds the
+    six inputs and the output of every layer's recurrence to bfloat16 and keeps everything else in float64 (the bonus
+    term after the op included): what a model computes whose op alone has bf16 I/O."""
     tokens = np.asarray(tokens)
     T = tokens.shape[0]
     if length is None:
@@ -108,7 +121,7 @@ def forward(params, tokens, state, length=None, new_starts=None):         # llm.
     for i in range(L):
         blk = _layer(params["blocks"], i)
         dx, s, v_first = time_mixing_seq(layer_norm(x, blk["ln1"]), state[i, 1:], v_first, blk["att"], length,
-                                         new_starts, H, S, i)
+                                         new_starts, H, S, i, op_io)
         state[i, 1:] = s
         x = x + dx
         dx, s0 = channel_mixing_seq(layer_norm(x, blk["ln2"]), state[i, :1], blk["ffn"], length, new_starts)

@@ -220,3 +220,33 @@ def test_channel_mix_without_token_shift_is_a_relu_squared_mlp(model):
     xk = tt(x + (prev - x) * ffn["x_k"])
     ref = F.linear(F.relu(F.linear(xk, tt(ffn["key"]["weight"]))) ** 2, tt(ffn["value"]["weight"])).numpy()
     np.testing.assert_allclose(out, ref, rtol=1e-10, atol=1e-12)
+
+
+def test_bf16_op_io_rounds_the_six_inputs_and_the_output_and_nothing_else(model, monkeypatch):
+    """forward(op_io="bf16"): the recurrence sees bf16-representable r, w, k, v, a, b (the same values as without the
+    option, rounded to nearest even), its output is rounded before the group norm, and the bonus term, the state and
+    every projection stay float64."""
+    from tests.inputs import bf16_round
+    spy = Spy(monkeypatch)
+    T, C = 11, 128
+    x = np.random.default_rng(9).standard_normal((T, C))
+    L, H, S = model["blocks"]["att"]["r_k"].shape
+    state = 0.1 * np.random.default_rng(10).standard_normal((1 + S, C))
+    att = att_of(model, 1)
+    exact = om.time_mixing_seq(x, state, x, att, T, np.zeros(T, bool), H, S, 1)
+    plain = spy.calls[-1]
+    rounded = om.time_mixing_seq(x, state, x, att, T, np.zeros(T, bool), H, S, 1, op_io="bf16")
+    seen = spy.calls[-1]
+    for n in "rwkvab":
+        np.testing.assert_array_equal(seen[n], bf16_round(plain[n]).astype(np.float64))
+        assert np.any(seen[n] != plain[n])
+    rel = lambda a, b: np.sqrt(np.mean((a - b) ** 2) / np.mean(b ** 2))
+    assert 1e-4 < rel(rounded[0], exact[0]) < 2e-2             # bf16 rounding of the op's I/O, nothing coarser
+    assert rel(rounded[1][1:], exact[1][1:]) < 2e-2 and np.array_equal(rounded[1][0], exact[1][0])
+    # with an output projection that reads the bonus term only (zero group-norm weight and bias), y does not depend on
+    # the op's output at all: the option must not touch that path
+    att0 = dict(att)
+    att0["ln_x"] = {"weight": np.zeros_like(att["ln_x"]["weight"]), "bias": np.zeros_like(att["ln_x"]["bias"])}
+    a0 = om.time_mixing_seq(x, state, x, att0, T, np.zeros(T, bool), H, S, 1)
+    b0 = om.time_mixing_seq(x, state, x, att0, T, np.zeros(T, bool), H, S, 1, op_io="bf16")
+    np.testing.assert_array_equal(a0[0], b0[0])
