@@ -29,7 +29,7 @@ B, T, H, N = 8, 4096, 32, 64
 # figures in profiles/), each with the sha1 prefix of the kernel source it was measured on: when the source has
 # changed since, `roofline.traffic` is null instead of a stale figure.
 MEASURED_TRAFFIC = {
-    "wkv7_fwd": (948.5e6, "wkv7_fwd.hip", "SHA_WKV7", "profiles/wkv7_fwd_B8_T4096_H32_bf16.md"),
+    "wkv7_fwd": (948.5e6, "wkv7_fwd.hip", "36b60ec7025c", "profiles/wkv7_fwd_B8_T4096_H32_bf16.md"),
     "wkv4_fwd": (4028.7e6, "wkv4.hip", "d83a0992a92e", "profiles/wkv4_fwd_B32_T4096_C2560_f32.md"),
     "wkv6_fwd": (688.5e6, "wkv6_fwd.hip", "SHA_WKV6", "profiles/wkv6_fwd_bwd_B16_T2048_H32_bf16.md"),
 }
@@ -186,7 +186,7 @@ def roofline(bytes_per_launch, kern_ms, traffic):
             "traffic": nbytes, "traffic_source": source, "kernel_ms": kern_ms, "algorithmic_bytes": bytes_per_launch}
 
 
-def power_probe(torch, fn, seconds=1.6):
+def power_probe(torch, fn, seconds=4.0):
     """Socket power while `fn` runs back to back: launches are queued for about `seconds`, `amd-smi` is read twice
     while the GPU works through them.  None where the tool is missing or prints nothing usable."""
     import shutil
@@ -219,16 +219,25 @@ def power_probe(torch, fn, seconds=1.6):
     per_call = e0.elapsed_time(e1) / 5 * 1e-3
     for _ in range(max(10, int(seconds / per_call))):
         fn()
-    time.sleep(0.5)
+    time.sleep(0.7)
     w1 = read(["metric", "-g", "0", "--power"], "SOCKET_POWER")
-    w2 = read(["metric", "-g", "0", "--power"], "SOCKET_POWER")
-    busy = not torch.cuda.current_stream().query()
+    busy1 = not torch.cuda.current_stream().query()
+    w2 = read(["metric", "-g", "0", "--power"], "SOCKET_POWER") if busy1 else None
+    busy2 = not torch.cuda.current_stream().query()
     torch.cuda.synchronize()
-    cap = read(["static", "-g", "0", "--limit"], "MAX_POWER")
+    cap = None
+    try:
+        txt = subprocess.run(["rocm-smi", "--showmaxpower"], capture_output=True, text=True, timeout=20).stdout
+        for line in txt.splitlines():
+            if "Max Graphics Package Power" in line:
+                cap = float(line.split(":")[-1])
+    except Exception:
+        pass
     if w1 is None and w2 is None:
         return None
-    return {"socket_w": [w1, w2], "cap_w": cap, "gpu_still_busy_after_reads": busy,
-            "how": "amd-smi metric --power, read twice while the forward kernel runs back to back"}
+    return {"socket_w": [w1 if busy1 else None, w2 if busy2 else None], "cap_w": cap,
+            "how": "amd-smi metric --power while the timed call runs back to back (a reading is kept only if the GPU "
+                   "was still busy after it)"}
 
 
 def bench_wkv7(torch, ops, args):
@@ -264,6 +273,8 @@ def bench_wkv7(torch, ops, args):
                           "note": "forward keeps the residual sa (fp16 beside bf16 I/O); backward = three sweeps (reverse, forward, reverse), " +
                                   ("sequential fp32 VALU kernels" if args.seq else "chunked MFMA kernels") +
                                   "; dsa and the decay-gradient terms pass through an fp32 workspace"}
+        if not args.no_power:
+            out["fwd_bwd"]["power"] = power_probe(torch, fwd_bwd)
     if not args.no_fp32:
         # the same shape with fp32 r/w/k/v/a/b/y: the chunked kernel on fp32 matrix instructions (or, with --seq, the
         # sequential kernel); 14 token tensors' worth of bytes against the same 8 TB/s
