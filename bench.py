@@ -186,45 +186,42 @@ def roofline(bytes_per_launch, kern_ms, traffic):
             "traffic": nbytes, "traffic_source": source, "kernel_ms": kern_ms, "algorithmic_bytes": bytes_per_launch}
 
 
-def power_probe(torch, fn, seconds=4.0):
-    """Socket power while `fn` runs back to back: launches are queued for about `seconds`, `amd-smi` is read twice
-    while the GPU works through them.  None where the tool is missing or prints nothing usable."""
+def power_probe(torch, fn, seconds=3.0):
+    """Socket power while `fn` runs back to back: the calling thread keeps launching while a second thread waits
+    `seconds` / 3 and reads `amd-smi` twice.  None where the tool is missing or prints nothing usable."""
     import shutil
     import subprocess
+    import threading
     if shutil.which("amd-smi") is None:
         return None
+    got = {"w": [], "done": False}
 
-    def read(args, key):
+    def read_power():
         try:
-            txt = subprocess.run(["amd-smi"] + args, capture_output=True, text=True, timeout=20).stdout
+            txt = subprocess.run(["amd-smi", "metric", "-g", "0", "--power"], capture_output=True, text=True, timeout=20).stdout
         except Exception:
             return None
         for line in txt.splitlines():
-            if key in line:
+            if "SOCKET_POWER" in line:
                 try:
                     return float(line.split(":")[1].split()[0])
                 except (IndexError, ValueError):
                     return None
         return None
 
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    for _ in range(20):
-        fn()
-    torch.cuda.synchronize()
-    e0.record()
-    for _ in range(5):
-        fn()
-    e1.record()
-    torch.cuda.synchronize()
-    per_call = e0.elapsed_time(e1) / 5 * 1e-3
-    for _ in range(max(10, int(seconds / per_call))):
-        fn()
-    time.sleep(0.7)
-    w1 = read(["metric", "-g", "0", "--power"], "SOCKET_POWER")
-    busy1 = not torch.cuda.current_stream().query()
-    w2 = read(["metric", "-g", "0", "--power"], "SOCKET_POWER") if busy1 else None
-    busy2 = not torch.cuda.current_stream().query()
-    torch.cuda.synchronize()
+    def reader():
+        time.sleep(seconds / 3.0)
+        got["w"].append(read_power())
+        got["w"].append(read_power())
+        got["done"] = True
+
+    th = threading.Thread(target=reader)
+    th.start()
+    while not got["done"]:
+        for _ in range(16):
+            fn()
+        torch.cuda.synchronize()          # keeps the launch queue short, so the loop ends soon after the readings
+    th.join()
     cap = None
     try:
         txt = subprocess.run(["rocm-smi", "--showmaxpower"], capture_output=True, text=True, timeout=20).stdout
@@ -233,11 +230,10 @@ def power_probe(torch, fn, seconds=4.0):
                 cap = float(line.split(":")[-1])
     except Exception:
         pass
-    if w1 is None and w2 is None:
+    if all(w is None for w in got["w"]):
         return None
-    return {"socket_w": [w1 if busy1 else None, w2 if busy2 else None], "cap_w": cap,
-            "how": "amd-smi metric --power while the timed call runs back to back (a reading is kept only if the GPU "
-                   "was still busy after it)"}
+    return {"socket_w": got["w"], "cap_w": cap,
+            "how": "amd-smi metric --power, read twice by a second thread while the timed call runs back to back"}
 
 
 def bench_wkv7(torch, ops, args):
@@ -293,6 +289,22 @@ def bench_wkv7(torch, ops, args):
         del x32
     if not args.no_power:
         out["power"] = power_probe(torch, fwd)
+    if args.occupancy_probe:
+        # The same kernel on 8, 4 and 2 of the 8 sequences (256, 128, 64 workgroups = CUs): launch time and socket power.
+        # Every workgroup does the same work in each case, so a launch time that grows with the number of busy CUs
+        # while the socket power approaches its cap shows the power limit (not the kernel's own pipeline) at work.
+        probe = []
+        for nb in (8, 4, 2):
+            xs = {n: (x[n][:nb].contiguous() if n != "dy" else None) for n in x}
+
+            def part():
+                return ops.wkv7_fwd(xs["r"], xs["w"], xs["k"], xs["v"], xs["a"], xs["b"], xs["s"], xs["length"],
+                                    xs["new_starts"], compat=True, want_sa=False)
+            _, kms = time_region(torch, part, 50, 5)
+            pw = power_probe(torch, part, seconds=3.0)
+            probe.append({"sequences": nb, "workgroups": nb * H, "kernel_ms": kms,
+                          "socket_w": None if pw is None else pw["socket_w"]})
+        out["occupancy_probe"] = probe
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
         out["cpu_baseline_sequential"] = cpu_baseline_sequential()
@@ -469,6 +481,8 @@ def main():
     ap.add_argument("--no-fp32", action="store_true", help="WKV7: skip the fp32-I/O leg")
     ap.add_argument("--seq", action="store_true", help="WKV7: force the sequential fp32 VALU kernel")
     ap.add_argument("--no-power", action="store_true", help="WKV7: skip the socket-power reading (amd-smi)")
+    ap.add_argument("--occupancy-probe", action="store_true",
+                    help="WKV7: also time the forward on 8, 4 and 2 sequences with a socket-power reading each")
     ap.add_argument("--no-secondary", action="store_true",
                     help="WKV7: skip the compact WKV6 / WKV4 records appended to the line")
     ap.add_argument("--no-stream-probe", action="store_true",
