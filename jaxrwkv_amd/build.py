@@ -19,8 +19,10 @@ FLAGS = [
 
 
 def build(verbose=True, jobs=None):
-    """Compiles every source to an object under ``jaxrwkv_amd/build/`` (in parallel) and links the shared library."""
+    """Compiles every source to an object under ``jaxrwkv_amd/build/`` (in parallel), checks the assembly of each
+    (``mfma_hazard``) and links the shared library."""
     from concurrent.futures import ThreadPoolExecutor
+    from . import mfma_hazard
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
     objdir = os.path.join(HERE, "build")
     os.makedirs(objdir, exist_ok=True)
@@ -37,9 +39,14 @@ def build(verbose=True, jobs=None):
             print(out)
 
     def compile_one(src):
-        obj = os.path.join(objdir, os.path.splitext(src)[0] + ".o")
-        run([hipcc] + compile_flags + ["-c", os.path.join(CSRC, src), "-o", obj])
-        return obj
+        stem = os.path.join(objdir, os.path.splitext(src)[0])
+        run([hipcc] + compile_flags + ["-c", os.path.join(CSRC, src), "-o", stem + ".o"])
+        # the same device code as assembly, for the check of MFMA pairings the compiler does not space out
+        run([hipcc] + [f for f in compile_flags if f != "-fPIC"] + ["-S", "--cuda-device-only", os.path.join(CSRC, src),
+                                                                   "-o", stem + ".s"])
+        with open(stem + ".s") as f:
+            mfma_hazard.check(f.read(), src)
+        return stem + ".o"
 
     jobs = jobs or min(8, os.cpu_count() or 1)
     with ThreadPoolExecutor(max_workers=jobs) as pool:

@@ -168,6 +168,18 @@ __device__ __forceinline__ void split2_keep(float x0, float x1, uint32_t& hi, ui
   lo = pack_rn(l0, l1);
 }
 
+// Keeps two matrix instructions of DIFFERENT opcodes apart when the second one accumulates on the first one's
+// result.  Measured on gfx950 with hipcc 7.2: v_mfma_f32_16x16x32_f16 D followed by v_mfma_f32_16x16x16_f16 D, A, B, D
+// reads a stale D in the first quarter of the wave (register 0 of lanes 0-15) when three or four other instructions
+// sit between the two, and the right one from five on; the compiler's hazard recogniser adds no wait states there
+// (it does for every other pairing the library has: same opcode, or a different destination).  Which distance a
+// build gets depends on instruction scheduling, so unrelated source changes switched the error on and off.  The
+// eight wait states here are the distance the compiler itself keeps between a matrix instruction and an ordinary
+// vector instruction that reads its result.  The asm takes the accumulator as an in/out operand, which pins it
+// between the two matrix instructions.  tests/test_mfma_hazard.py checks the distance in the compiled code of every
+// kernel.
+__device__ __forceinline__ void mfma_shape_fence(f32x4_t& acc) { asm volatile("s_nop 7" : "+v"(acc)); }
+
 // First statement of a rarely taken, wave-uniform branch (resets inside a chunk, the partial last chunk, the chunk
 // of token length-1): keeps the compiler from turning the branch into selects that every chunk would execute.
 __device__ __forceinline__ void rare_path() { asm volatile("" ::: "memory"); }

@@ -462,11 +462,13 @@ __device__ __forceinline__ bool consume(Consumer& C, Ops& o, const Slot* __restr
                     pack_h(C.S[2 * j + 1][0], C.S[2 * j + 1][1]), pack_h(C.S[2 * j + 1][2], C.S[2 * j + 1][3])};
   f32x4_t W = zero4;              // [token 4g+i][value n], two interleaved accumulation chains
   f32x4_t Y = mfma_h16(o.KrLo, o.vv, zero4);    // the low part of Mkr^T V^T: no state in it, off the critical path
+  mfma_shape_fence(Y);                          // a K = 16 result enters a K = 32 chain
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     W = mfma_h(o.aq[0][j], Sh[j], W);
     Y = mfma_h(o.aq[1][j], Sh[j], Y);
   }
+  mfma_shape_fence(W);                          // a K = 32 result enters a K = 16 instruction: the pairing that fails
   W = mfma_h16(o.Ka, o.vv, W);                  // W += Mka^T V^T
   const f32x4_t SA = mfma_h16(o.P, pack_h4(W), zero4);
   const u32x2_t sp = pack_h4(SA);
