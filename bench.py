@@ -287,6 +287,36 @@ def bench_wkv7(torch, ops, args):
                           "mfma_frac": None if args.seq else fp32_mfma_flops(tokens) / (k32 * 1e-3) / 1e12 / 157.3,
                           "kernel": "sequential fp32 VALU" if args.seq else "chunked, v_mfma_f32_16x16x4_f32 (fp32 operands)"}
         del x32
+    if not args.no_placement and not args.seq:
+        # The same two measurements with the seven input arrays copied to addresses 0, 128, ..., 768 bytes past a 1 KiB
+        # boundary instead of all on 2 MiB boundaries (where torch's allocator puts them, and where `value` and
+        # `fwd_bwd` above are measured): rows of different arrays at the same (token, head) then no longer compete for
+        # the same part of the memory system.  A caller that owns the placement of its operands gets these figures.
+        xp = dict(x)
+        for i, n in enumerate(("r", "w", "k", "v", "a", "b", "dy")):
+            xp[n] = ops._empty_phased(tuple(x[n].shape), x[n].dtype, x[n].device, i)
+            xp[n].copy_(x[n])
+
+        def fwd_p():
+            return ops.wkv7_fwd(xp["r"], xp["w"], xp["k"], xp["v"], xp["a"], xp["b"], xp["s"], xp["length"],
+                                xp["new_starts"], compat=True, want_sa=False)
+
+        def fwd_bwd_p():
+            new_s, y, sa = ops.wkv7_fwd(xp["r"], xp["w"], xp["k"], xp["v"], xp["a"], xp["b"], xp["s"], xp["length"],
+                                        xp["new_starts"], compat=True, want_sa=True)
+            return ops.wkv7_bwd(xp["r"], xp["w"], xp["k"], xp["v"], xp["a"], xp["b"], xp["s"], xp["length"],
+                                xp["new_starts"], xp["dy"], sa, None, compat=True)
+        _, kp = time_region(torch, fwd_p, max(10, args.steps // 2), 3)
+        rec = {"inputs_of_value": "every input array on a 2 MiB boundary (torch's allocator); outputs, gradients and "
+                                  "workspace arrays at their own 128-byte phases (the operators place them)",
+               "inputs_staggered": {"kernel_ms": kp, "tokens_per_s": tokens / (kp * 1e-3),
+                                    "hbm_frac": fwd_bytes / (kp * 1e-3) / 1e9 / HBM_PEAK_GBS}}
+        if not args.no_bwd:
+            n4 = max(10, args.steps // 4)
+            wall4, _ = time_region(torch, fwd_bwd_p, n4, 2)
+            rec["inputs_staggered"]["fwd_bwd_ms"] = 1e3 * wall4 / n4
+        out["placement"] = rec
+        del xp
     if not args.no_power:
         out["power"] = power_probe(torch, fwd)
     if args.occupancy_probe:
@@ -480,6 +510,7 @@ def main():
     ap.add_argument("--no-bwd", action="store_true")
     ap.add_argument("--no-fp32", action="store_true", help="WKV7: skip the fp32-I/O leg")
     ap.add_argument("--seq", action="store_true", help="WKV7: force the sequential fp32 VALU kernel")
+    ap.add_argument("--no-placement", action="store_true", help="skip the run with the inputs at staggered addresses")
     ap.add_argument("--no-power", action="store_true", help="WKV7: skip the socket-power reading (amd-smi)")
     ap.add_argument("--occupancy-probe", action="store_true",
                     help="WKV7: also time the forward on 8, 4 and 2 sequences with a socket-power reading each")

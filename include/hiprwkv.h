@@ -19,6 +19,16 @@
  *   length                   (B,) uint32, may be NULL (= T)
  *   new_starts               (B,T) one byte per token (0/1), may be NULL (= none)
  * The recurrence always runs in fp32 whatever the io/state dtypes are.
+ *
+ * Placement of the token tensors.  The kernels touch the rows of all token tensors of a call at the same
+ * (token, head) together.  When the tensors' base addresses are congruent modulo 1 KiB (two large allocations
+ * of a caching allocator usually are: both start on 2 MiB boundaries) those rows compete for the same part of
+ * the memory system.  Measured on MI355X, WKV7 at B8 T4096 H32 bf16, forward with its residual / forward +
+ * backward: 303 / 1619 us with every tensor on a 2 MiB boundary; 284 / 1535 us with only the outputs, the
+ * gradients and the workspace arrays moved; 265 / 1469 us with each tensor, the inputs included, at its own
+ * multiple of 128 bytes past a 1 KiB boundary (0, 128, ..., 896).  Offsets that are multiples of 1 KiB change
+ * nothing.  A caller that owns the placement of its operands should stagger them that way; the library does
+ * it for the arrays inside `workspace`, and the Python operators do it for every tensor they allocate.
  */
 #ifndef HIPRWKV_H_
 #define HIPRWKV_H_
@@ -121,7 +131,7 @@ int hiprwkv_wkv7_step(hiprwkv_stream stream, int io_dtype, int state_dtype,
                       const uint32_t* length, const uint8_t* new_starts,
                       void* out, void* new_s, int64_t new_s_batch_stride, unsigned flags);
 
-/* Bytes of scratch hiprwkv_wkv7_bwd needs for this shape. */
+/* Bytes of scratch hiprwkv_wkv7_bwd needs for this shape: three fp32 (B,T,H,N) arrays plus 1 KiB each (see "Placement"). */
 size_t hiprwkv_wkv7_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t N);
 
 /* Replaces ffi target "wkv7-bwd-{fp32,bf16}": operands w,r,k,v,a,b,s,length,new_starts,

@@ -29,6 +29,19 @@ bool dtype_ok(int d) { return d == HIPRWKV_F32 || d == HIPRWKV_BF16; }
 
 size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
+// Rows of different (B,T,H,N) arrays at the same (token, head) are accessed together; arrays whose base addresses are
+// congruent modulo 1 KiB then compete for the same part of the memory system (measured on MI355X: the backward sweeps
+// that read and write the workspace arrays lose 5-10 % when everything starts on a 2 MiB boundary, and offsets that
+// are multiples of 1 KiB change nothing).  The workspace arrays therefore start at their own 128-byte step past the
+// phase of the first operand.
+constexpr size_t PHASE_BYTES = 128, PHASE_SPAN = 1024;
+char* at_phase(char* p, const void* like, unsigned steps) {
+  const uintptr_t want = (reinterpret_cast<uintptr_t>(like) + steps * PHASE_BYTES) % PHASE_SPAN / PHASE_BYTES * PHASE_BYTES;
+  const uintptr_t at = reinterpret_cast<uintptr_t>(p);
+  const uintptr_t up = (at + 15) & ~(uintptr_t)15;
+  return reinterpret_cast<char*>(up + (want + PHASE_SPAN - up % PHASE_SPAN) % PHASE_SPAN);
+}
+
 int check_matrix_shape(const char* op, int io_dtype, int state_dtype, int64_t B, int64_t T, int64_t H, int64_t N) {
   if (!dtype_ok(io_dtype) || !dtype_ok(state_dtype)) return fail(HIPRWKV_EINVAL, "%s: dtype must be HIPRWKV_F32 or HIPRWKV_BF16", op);
   if (N != 64) return fail(HIPRWKV_EINVAL, "%s: head size N=%lld not supported (kernels are built for N=64)", op, (long long)N);
@@ -203,7 +216,7 @@ int hiprwkv_wkv7_step(hiprwkv_stream stream, int io_dtype, int state_dtype, int6
 }
 
 size_t hiprwkv_wkv7_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t N) {
-  return 3 * align256((size_t)B * T * H * N * sizeof(float));
+  return 3 * (align256((size_t)B * T * H * N * sizeof(float)) + PHASE_SPAN);
 }
 
 int hiprwkv_wkv7_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64_t B, int64_t T, int64_t H, int64_t N,
@@ -232,11 +245,11 @@ int hiprwkv_wkv7_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64
   A.status = status_word();
   A.gy = gy; A.sa_in = sa; A.gs_out = gs_out;
   A.gw = gw; A.gr = gr; A.gk = gk; A.gv = gv; A.ga = ga; A.gb = gb; A.gs = gs;
-  const size_t one = need / 3;
+  const size_t one = need / 3 - PHASE_SPAN;
   char* ws = static_cast<char*>(workspace);
-  A.dsa = reinterpret_cast<float*>(ws);
-  A.e2 = reinterpret_cast<float*>(ws + one);
-  A.e3 = reinterpret_cast<float*>(ws + 2 * one);
+  A.dsa = reinterpret_cast<float*>(at_phase(ws, r, 3));
+  A.e2 = reinterpret_cast<float*>(at_phase(reinterpret_cast<char*>(A.dsa) + one, r, 5));
+  A.e3 = reinterpret_cast<float*>(at_phase(reinterpret_cast<char*>(A.e2) + one, r, 7));
   // Three sweeps: A (reverse) -> gv, dsa, gs; B (forward) -> gr, ga, e2, e3 (the chunked B: their sum shifted by a
   // token, in e2); C (reverse) -> gk, gb, gw.
   // bf16 I/O runs all three on the chunked MFMA kernels.
@@ -311,7 +324,7 @@ int hiprwkv_wkv6_step(hiprwkv_stream stream, int io_dtype, int state_dtype, int6
 }
 
 size_t hiprwkv_wkv6_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t N) {
-  return align256((size_t)B * T * H * N * sizeof(float)) + align256((size_t)B * H * N * sizeof(float));
+  return align256((size_t)B * T * H * N * sizeof(float)) + PHASE_SPAN + align256((size_t)B * H * N * sizeof(float));
 }
 
 int hiprwkv_wkv6_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64_t B, int64_t T, int64_t H, int64_t N,
@@ -341,8 +354,8 @@ int hiprwkv_wkv6_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64
   A.gy = gy; A.gs_out = gs_out;
   A.gr = gr; A.gk = gk; A.gv = gv; A.gw = gw; A.gu = gu; A.gs = gs;
   char* ws = static_cast<char*>(workspace);
-  A.er = reinterpret_cast<float*>(ws);
-  A.eI = reinterpret_cast<float*>(ws + align256((size_t)B * T * H * N * sizeof(float)));
+  A.er = reinterpret_cast<float*>(at_phase(ws, r, 5));
+  A.eI = reinterpret_cast<float*>(reinterpret_cast<char*>(A.er) + align256((size_t)B * T * H * N * sizeof(float)));
   // Two sweeps: F (forward) -> gr, gu, er, eI; R (reverse) -> gk, gv, gw, gs.  bf16 I/O runs them on the chunked
   // MFMA kernels.
   hipStream_t st = static_cast<hipStream_t>(stream);

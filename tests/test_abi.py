@@ -58,7 +58,8 @@ def test_argument_validation_without_gpu():
     assert rc == -3 and b"needed" in lib.hiprwkv_last_error()
     rc = lib.hiprwkv_wkv4_fwd_ckpt(null, 0, 0, 17, 64, *([ok] * 5), null, null, ok, ok, ok, 1 << 20, 0)
     assert rc == -1
-    assert lib.hiprwkv_wkv7_bwd_workspace_bytes(2, 16, 2, 64) == 3 * 2 * 16 * 2 * 64 * 4
+    # three fp32 (B,T,H,N) arrays, each with 1 KiB of room to start at its own 128-byte phase
+    assert lib.hiprwkv_wkv7_bwd_workspace_bytes(2, 16, 2, 64) == 3 * (2 * 16 * 2 * 64 * 4 + 1024)
     # the decode step on a packed state: at most 8 tokens, batch strides of at least one state and 16-byte multiples
     step = lambda T, s_stride, o_stride, st=1: lib.hiprwkv_wkv7_step(null, 1, st, 2, T, 2, 64, *([ok] * 7), s_stride, null,
                                                                    null, ok, ok, o_stride, 0)
@@ -201,3 +202,24 @@ def test_flag_bits_are_validated_without_gpu():
         out = subprocess.run([sys.executable, "-c", code], cwd=ROOT, env=env, capture_output=True, text=True, timeout=120)
         assert out.returncode == 0, out.stderr
         assert out.stdout.startswith("-1 ") and want in out.stdout, out.stdout
+
+
+def test_phased_allocation_gives_the_asked_address_phase():
+    """The operators place the large arrays they allocate at distinct 128-byte steps past a 1 KiB boundary
+    (jaxrwkv_amd/ops.py); small ones are allocated plainly.  Runs on CPU tensors: only addresses are looked at."""
+    import torch
+    from jaxrwkv_amd import ops
+    ref = torch.empty((2, 512, 8, 64), dtype=torch.bfloat16)            # 1 MiB
+    seen = set()
+    for steps in range(1, 9):
+        t = ops._empty_like_phased(ref, steps)
+        assert t.shape == ref.shape and t.dtype == ref.dtype and t.is_contiguous()
+        assert (ops._phase(t) - ops._phase(ref)) % 8 == steps % 8
+        assert t.data_ptr() % 16 == 0
+        seen.add(ops._phase(t))
+        t.fill_(1.0)                                                    # the whole view is writable memory
+    assert len(seen) == 8
+    small = ops._empty_phased((4, 1, 8, 64), torch.float32, "cpu", 3)
+    assert small.shape == (4, 1, 8, 64) and small._base is None
+    f16 = ops._empty_phased((2, 512, 8, 64), torch.float16, "cpu", 5)
+    assert ops._phase(f16) == 5 and f16.dtype == torch.float16
