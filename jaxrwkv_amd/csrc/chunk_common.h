@@ -274,13 +274,12 @@ __device__ __forceinline__ ChunkFlags chunk_flags_of(const uint8_t* ns, uint32_t
   F.ns = ns != nullptr ? (uint32_t)(__ballot(mine != 0) & ((1ull << have) - 1ull)) : 0u;
   return F;
 }
-// Without new_starts (a null pointer is legal) nothing is loaded: the branch is uniform, the pointer is a kernel
-// argument.
-__device__ __forceinline__ ChunkFlags chunk_flags(const uint8_t* ns, unsigned flags, int64_t T, int64_t b, int64_t c0,
-                                                  int64_t L, int lane) {
-  uint32_t mine = 0u;
-  if (ns != nullptr) mine = chunk_flag_fetch(ns, T, b, c0, lane);
-  return chunk_flags_of(ns, mine, flags, T, c0, L);
+// The producers fetch this byte one step ahead, before the operands of the same chunk (in that order: waiting for it
+// then leaves the operand loads in flight); fetched at the top of the step it would cost every step a full memory
+// round trip.  Without new_starts (a null pointer is legal) nothing is loaded: the branch is uniform, the pointer is a
+// kernel argument.
+__device__ __forceinline__ uint32_t chunk_flag_prefetch(const uint8_t* ns, int64_t T, int64_t b, int64_t c0, int lane) {
+  return ns != nullptr ? chunk_flag_fetch(ns, T, b, c0, lane) : 0u;
 }
 
 // Selection operands that turn an MFMA into a transposer: against an A operand whose k-slot (g, jj) stands for key

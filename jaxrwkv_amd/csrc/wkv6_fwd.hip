@@ -498,15 +498,22 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv6_fwd_kernel(Wkv6Args
   } else {
     const int p = wave - NCONS;
     Raw raw;
-    if (p < nch) load_raw(raw, A, b, h, (int64_t)p * CK, lane);
+    uint32_t ns_mine = 0u;      // this lane's new_starts byte of the chunk loaded next: fetched a step ahead, like the operands
+    if (p < nch) {
+      ns_mine = chunk_flag_prefetch(A.ns, A.T, b, (int64_t)p * CK, lane);
+      load_raw(raw, A, b, h, (int64_t)p * CK, lane);
+    }
     for (int j = p; j < nch; j += NPROD) {
       const int64_t c0 = (int64_t)j * CK;
-      const ChunkFlags F = chunk_flags(A.ns, A.flags, A.T, b, c0, L, lane);
+      const ChunkFlags F = chunk_flags_of(A.ns, ns_mine, A.flags, A.T, c0, L);
       const int si = j % RING;
       if (j >= RING && !wait_consumed_lazy(sy, si, j - RING + 1, lane)) break;
       mask_raw(raw, F.nvalid, lane);
       produce(lane, raw, F, ulds, &slots[si], snapslot, events_word(A.status));
-      if (j + NPROD < nch) load_raw(raw, A, b, h, c0 + (int64_t)NPROD * CK, lane);
+      if (j + NPROD < nch) {
+        ns_mine = chunk_flag_prefetch(A.ns, A.T, b, c0 + (int64_t)NPROD * CK, lane);
+        load_raw(raw, A, b, h, c0 + (int64_t)NPROD * CK, lane);
+      }
       if ((A.flags & FLAG_DROP_PUBLISH) && j + 1 == nch) break;
       // the release orders this wave's LDS writes before the sequence number
       if (lane == 0) __hip_atomic_store(&sy->ready[si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);

@@ -521,16 +521,23 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_bwd_b_kernel(
     P.lane = lane;
     make_sel(P.sel, lane);
     Raw raw;
-    if (p < nch) load_raw(raw, A, b, h, (int64_t)p * CK, lane);
+    uint32_t ns_mine = 0u;      // this lane's new_starts byte of the chunk loaded next: fetched a step ahead, like the operands
+    if (p < nch) {
+      ns_mine = chunk_flag_prefetch(A.ns, A.T, b, (int64_t)p * CK, lane);
+      load_raw(raw, A, b, h, (int64_t)p * CK, lane);
+    }
     for (int c = p; c < nch; c += NPROD) {
       const int64_t c0 = (int64_t)c * CK;
-      ChunkFlags F = chunk_flags(A.ns, A.flags, A.T, b, c0, L, lane);
+      ChunkFlags F = chunk_flags_of(A.ns, ns_mine, A.flags, A.T, c0, L);
       if (!inject) F.snap = -1;
       const int si = c % RING;
       Slot* slot = &slots[si];
       if (c >= RING && !wait_consumed(sy, si, c - RING + 1, lane)) break;
       produce(P, raw, F, slot, snapslot, events_word(A.status));
-      if (c + NPROD < nch) load_raw(raw, A, b, h, c0 + NPROD * CK, lane);
+      if (c + NPROD < nch) {
+        ns_mine = chunk_flag_prefetch(A.ns, A.T, b, c0 + NPROD * CK, lane);
+        load_raw(raw, A, b, h, c0 + NPROD * CK, lane);
+      }
       if ((A.flags & FLAG_DROP_PUBLISH) && c + 1 == nch) break;
       // the release orders this wave's LDS writes before the sequence number
       if (lane == 0) __hip_atomic_store(&sy->ready[si], c + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
