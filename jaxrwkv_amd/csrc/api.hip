@@ -216,7 +216,9 @@ int hiprwkv_wkv7_step(hiprwkv_stream stream, int io_dtype, int state_dtype, int6
 }
 
 size_t hiprwkv_wkv7_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t N) {
-  return 3 * (align256((size_t)B * T * H * N * sizeof(float)) + PHASE_SPAN);
+  // three fp32 arrays with one value per token and key; the second one is kept per chunk of 16 tokens (f_record)
+  const size_t tokens = (size_t)((T + 15) / 16) * 16;
+  return 3 * (align256((size_t)B * tokens * H * N * sizeof(float)) + PHASE_SPAN);
 }
 
 int hiprwkv_wkv7_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64_t B, int64_t T, int64_t H, int64_t N,

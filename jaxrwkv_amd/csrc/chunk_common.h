@@ -180,6 +180,25 @@ __device__ __forceinline__ void split2_keep(float x0, float x1, uint32_t& hi, ui
 // kernel.
 __device__ __forceinline__ void mfma_shape_fence(f32x4_t& acc) { asm volatile("s_nop 7" : "+v"(acc)); }
 
+// Last statement of the producers' branch of a kernel: "uses" every register that the producers load into from global
+// memory.  Both roles live in one function, and after the compiler has arranged the control flow the consumers' code
+// is, on paper, reachable from the end of the producers'.  Its pass that places the waits for memory operations then
+// believes that the registers of the producers' last loads may still be awaited when the consumers' code runs, and
+// guards their first reuse there -- inside the consumers' main loop -- with a full `s_waitcnt vmcnt(0)`, which at run
+// time waits for the consumer wave's own recent stores and loads in every step (seen in the reverse sweep C of the
+// WKV7 backward pass: a memory round trip per chunk on the critical path).  The empty asm statements make the
+// compiler wait for those loads here, where nothing is in flight any more, which clears that state.  (A
+// `__builtin_amdgcn_s_waitcnt` at the start of the consumers' branch does not do it: the pass removes it.)
+template <class R>
+__device__ __forceinline__ void retire_loads(const R& x, uint32_t flag_byte) {
+  constexpr int N = sizeof(R) / 4;
+  struct Words { uint32_t w[N]; };
+  const Words v = __builtin_bit_cast(Words, x);
+#pragma unroll
+  for (int i = 0; i < N; ++i) asm volatile("" ::"v"(v.w[i]));
+  asm volatile("" ::"v"(flag_byte));
+}
+
 // First statement of a rarely taken, wave-uniform branch (resets inside a chunk, the partial last chunk, the chunk
 // of token length-1): keeps the compiler from turning the branch into selects that every chunk would execute.
 __device__ __forceinline__ void rare_path() { asm volatile("" ::: "memory"); }
@@ -280,6 +299,16 @@ __device__ __forceinline__ ChunkFlags chunk_flags_of(const uint8_t* ns, uint32_t
 // kernel argument.
 __device__ __forceinline__ uint32_t chunk_flag_prefetch(const uint8_t* ns, int64_t T, int64_t b, int64_t c0, int lane) {
   return ns != nullptr ? chunk_flag_fetch(ns, T, b, c0, lane) : 0u;
+}
+
+// The fp32 workspace that the forward sweep of the WKV7 backward pass leaves for the reverse sweep after it (one value
+// per token and key) is laid out for the waves that write and read it, not by token: per (sequence, head, chunk,
+// consumer wave q) one record of 64 x 4 floats, lane (n, g) owning the four tokens 4g..4g+3 at key 16q + n.  Both
+// sweeps hold their per-token results in exactly that register layout, so each lane moves its record entry with one
+// 16-byte access (1 KiB contiguous per wave) instead of four scattered 4-byte ones.
+constexpr int F_REC = 64 * 4;       // floats per record
+__device__ __forceinline__ size_t f_record(int64_t b, int64_t h, int64_t H, int nch, int c, int q) {
+  return ((((size_t)b * H + h) * nch + c) * NCONS + q) * F_REC;
 }
 
 // Selection operands that turn an MFMA into a transposer: against an A operand whose k-slot (g, jj) stands for key

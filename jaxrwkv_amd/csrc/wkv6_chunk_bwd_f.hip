@@ -441,6 +441,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv6_chunk_bwd_f_kernel(
       if ((A.flags & FLAG_DROP_PUBLISH) && c + 1 == nch) break;
       if (lane == 0) __hip_atomic_store(&sy->ready[si], c + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
+    retire_loads(raw, ns_mine);
     // du of this producer's tokens: sum over the 16 token lanes of a row, one writer per key
 #pragma unroll
     for (int e = 0; e < 16; ++e) {

@@ -659,6 +659,7 @@ __global__ __launch_bounds__(64 * (NCONS_R + NPROD)) void wkv6_chunk_bwd_r_kerne
       if ((A.flags & FLAG_DROP_PUBLISH) && j + 1 == nch) break;
       if (lane == 0) __hip_atomic_store(&sy->ready[si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
+    retire_loads(raw, ns_mine);
   }
   __syncthreads();
   if (head_broken(sy, A.status)) {

@@ -648,6 +648,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_bwd_a_kernel(Wkv7Ar
       // the release orders this wave's LDS writes before the sequence number
       if (lane == 0) __hip_atomic_store(&sy->ready[si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
+    retire_loads(raw, ns_mine);
   }
   __syncthreads();
   if (head_broken(sy, A.status)) {

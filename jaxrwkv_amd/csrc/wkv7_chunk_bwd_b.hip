@@ -314,7 +314,7 @@ struct Consumer {
 
 struct OutCursor {
   char *gr, *ga;       // bf16 outputs at (b, c0, h, 0)
-  char* ef;            // fp32 workspace at the same place
+  float* ef;           // this wave's record of the chunk in the fp32 workspace (f_record)
   size_t tok_bytes;    // bytes between consecutive tokens in the bf16 arrays (twice that in the fp32 ones)
   uint32_t voff;       // lane part of the address, in elements: (4g * H) * 64 + key
 };
@@ -456,14 +456,15 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
     if (full || 4 * g + i < nvalid) {
       *reinterpret_cast<uint16_t*>(oc.gr + lo * 2 + i * oc.tok_bytes) = odr[i];
       *reinterpret_cast<uint16_t*>(oc.ga + lo * 2 + i * oc.tok_bytes) = oda[i];
-      // token 15 of a full chunk that is not the last one waits for the next chunk (below)
-      if (i < 3 || g < 3 || last) *reinterpret_cast<float*>(oc.ef + lo * 4 + 2 * i * oc.tok_bytes) = f[i];
     }
   }
-  if (!first && g == 0)
-    *reinterpret_cast<float*>(oc.ef + lo * 4 - 2 * oc.tok_bytes) = open_prev + (follows(0) ? e2[0] : 0.f);
+  // The whole record entry at once.  Token 15 of a chunk that is not the last one is still open: its entry (lanes
+  // g = 3, element 3) is a placeholder until the next chunk overwrites it below; both stores come from this wave, to
+  // the same address, in program order.  Entries of tokens beyond the sequence are never used.
+  *reinterpret_cast<float4*>(oc.ef + 4 * lane) = make_float4(f[0], f[1], f[2], f[3]);
+  if (!first && g == 0) (oc.ef - NCONS * F_REC)[4 * (48 + n) + 3] = open_prev + (follows(0) ? e2[0] : 0.f);
   oc.gr += CK * oc.tok_bytes; oc.ga += CK * oc.tok_bytes;
-  oc.ef += 2 * CK * oc.tok_bytes;
+  oc.ef += NCONS * F_REC;
 }
 
 }  // namespace
@@ -504,7 +505,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_bwd_b_kernel(
     const size_t el0 = (((size_t)b * A.T) * A.H + h) * 64;
     oc.gr = reinterpret_cast<char*>(A.gr) + el0 * 2;
     oc.ga = reinterpret_cast<char*>(A.ga) + el0 * 2;
-    oc.ef = reinterpret_cast<char*>(A.e2) + el0 * 4;
+    oc.ef = A.e2 + f_record(b, h, A.H, nch, 0, wave);
     oc.voff = (uint32_t)((4 * g) * (int)A.H * 64 + 16 * wave + n);
     const int csnap = (L >= 1 && inject) ? (int)((L - 1) / CK) : -1;
     for (int c = 0; c < nch; ++c) {
@@ -542,12 +543,15 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_bwd_b_kernel(
       // the release orders this wave's LDS writes before the sequence number
       if (lane == 0) __hip_atomic_store(&sy->ready[si], c + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
+    // (no retire_loads here: measured, this sweep is 5 % slower with it -- its producers are the bottleneck, and
+    // keeping their operand registers alive to the end of the loop costs them more than the consumers gain)
   }
   __syncthreads();
   if (head_broken(sy, A.status)) {
     poison_token_rows(A.gr, 2, b, h, A.T, A.H);
     poison_token_rows(A.ga, 2, b, h, A.T, A.H);
-    poison_token_rows(A.e2, 4, b, h, A.T, A.H);
+    for (size_t i = threadIdx.x; i < (size_t)nch * NCONS * F_REC; i += blockDim.x)
+      A.e2[f_record(b, h, A.H, nch, 0, 0) + i] = __uint_as_float(0x7fc00000u);
   }
 }
 

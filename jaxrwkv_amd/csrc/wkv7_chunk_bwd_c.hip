@@ -32,7 +32,7 @@ namespace {
 using namespace chunk;
 
 constexpr int NPROD = 4;          // producer waves; producer p owns steps p, p + NPROD, ...
-constexpr int RING = 5;           // slots in flight (a slot is 30 KB)
+constexpr int RING = 3;           // slots in flight (a slot is 40 KB)
 constexpr int ES = 68;            // row stride (floats) of the fp32 [token][key] array: conflict-free column reads
 
 // "lane-indexed" arrays hold, for every lane of the producer, the bytes the same lane of a consumer loads:
@@ -49,6 +49,15 @@ struct __attribute__((aligned(16))) Slot {
   uint4 Nk[2][64];             // [hi|lo] of {dsa_s.v_t (s > t), dy_s.v_t (s >= t)}, lane-indexed: A operand row t, k-slots s
   uint4 Nb[2][64];             // [hi|lo] of {dsa_s.sa_t (s > t), dy_s.sa_t (s >= t)}
   float Einv[CK][ES];          // 1/E_t per key
+  // What the decay-gradient recursion reads per token and key, brought in by the producers with the chunk's other
+  // operands: the k, b and w rows as they are in memory (bf16, natural key order) and the chunk's four records of
+  // the fp32 workspace that the forward sweep left (f_record), one per consumer wave.  Fetched by the consumers
+  // themselves, one chunk ahead, these values arrived late (behind the producers' deep queues a load takes several
+  // chunk times), and where the compiler put the waits depended on details of the source.  The slot grows to 40 KB
+  // and the ring shrinks from five slots to three; measured on MI355X the sweep takes the same time when the
+  // outputs sit at their own address phases and 8 % less when every array starts on a 2 MiB boundary.
+  uint16_t KBW[3][CK][RS];
+  float4 F[NCONS][64];
   float gamma[64];             // E at the chunk end
   int snap;                    // -1, or the in-chunk index of token length-1
   int keep_end;                // the cotangent of later chunks reaches the chunk start (no reset in the chunk)
@@ -67,10 +76,18 @@ struct Raw {
   uint4 w[2], r[2], a[2], v[2], dy[2];
   uint4 sa[2];             // the forward residual, fp16
   float4 dsa[2][2];
+  uint4 k[2], b[2];        // passed on to the consumers as they are
+  float4 f[NCONS];         // lane l: entry l of each consumer wave's record of this chunk
 };
 
 __device__ __forceinline__ void load_raw(Raw& x, const Wkv7Args& A, int64_t b, int64_t h, int64_t c0, int lane) {
   const int t = lane & 15, g = lane >> 4;
+  {
+    const int nch = (int)((A.T + CK - 1) / CK);
+    const float4* rec = reinterpret_cast<const float4*>(A.e2 + f_record(b, h, A.H, nch, (int)(c0 / CK), 0));
+#pragma unroll
+    for (int q = 0; q < NCONS; ++q) x.f[q] = rec[64 * q + lane];
+  }
   if (c0 + t < A.T) {
     const size_t el = (((size_t)b * A.T + c0 + t) * A.H + h) * 64 + 8 * g;
     auto ld = [&](const void* p, uint4 (&o)[2]) {
@@ -85,11 +102,12 @@ __device__ __forceinline__ void load_raw(Raw& x, const Wkv7Args& A, int64_t b, i
     };
     ld(A.w, x.w); ld(A.r, x.r); ld(A.a, x.a); ld(A.v, x.v); ld(A.gy, x.dy);
     ld(A.sa_in, x.sa); ld32(A.dsa, x.dsa);
+    ld(A.k, x.k); ld(A.b, x.b);
   } else {
     const uint4 z = make_uint4(0, 0, 0, 0);
     const float4 zf = make_float4(0.f, 0.f, 0.f, 0.f);
     x.w[0] = x.w[1] = x.r[0] = x.r[1] = x.a[0] = x.a[1] = x.v[0] = x.v[1] = x.dy[0] = x.dy[1] = z;
-    x.sa[0] = x.sa[1] = z;
+    x.sa[0] = x.sa[1] = x.k[0] = x.k[1] = x.b[0] = x.b[1] = z;
     x.dsa[0][0] = x.dsa[0][1] = x.dsa[1][0] = x.dsa[1][1] = zf;
   }
 }
@@ -152,6 +170,15 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
   auto plain_pack = [&](const f32x4_t d) { return make_uint2(pack_exact(d[0], d[1]), pack_exact(d[2], d[3])); };
   auto join = [&](const uint2 hi, const uint2 lo) { return make_uint4(hi.x, hi.y, lo.x, lo.y); };
 
+  // the consumers' per-token scalars, as loaded (rows beyond the sequence are zero)
+#pragma unroll
+  for (int hf = 0; hf < 2; ++hf) {
+    *reinterpret_cast<uint4*>(&slot->KBW[0][t][32 * hf + 8 * g]) = x.k[hf];
+    *reinterpret_cast<uint4*>(&slot->KBW[1][t][32 * hf + 8 * g]) = x.b[hf];
+    *reinterpret_cast<uint4*>(&slot->KBW[2][t][32 * hf + 8 * g]) = x.w[hf];
+  }
+#pragma unroll
+  for (int q = 0; q < NCONS; ++q) slot->F[q][lane] = x.f[q];
   // Gram tiles over the values, accumulator layout [row m = s][column n = t]
   f32x4_t Nsv = zero4, Nyv = zero4, Nss = zero4, Nys = zero4;
 #pragma unroll
@@ -311,44 +338,14 @@ struct Consumer {
   int q, lane;
 };
 
-// Per-token scalars at (token 4g+i, key 16q+n) that the decay-gradient recursion reads from global memory,
-// fetched one chunk ahead.
-struct Pre {
-  float f[4];                  // e3_t + e2_{t+1}, left by sweep B
-  uint16_t k[4], b[4], w[4];   // bf16 bits, widened where they are used: nothing waits for the loads before that
-};
-
 struct Cursor {
-  const char* ef;              // fp32 workspace at (b, c0, h, 0)
-  const char *k, *b, *w;       // bf16 inputs at the same place
-  char *gk, *gb, *gw;          // bf16 outputs
+  char *gk, *gb, *gw;          // bf16 outputs at (b, c0, h, 0)
   size_t tok_bytes;            // bytes between consecutive tokens in the bf16 arrays (twice that in the fp32 ones)
   uint32_t voff;               // lane part of the address, in elements: (4g * H) * 64 + key
 };
 
-__device__ __forceinline__ void prefetch(Pre& p, const Cursor& cu, int nvalid, int g) {
-  const rsrc_t rf = make_rsrc(cu.ef), rk = make_rsrc(cu.k), rb = make_rsrc(cu.b), rw = make_rsrc(cu.w);
-  const int o2 = (int)(cu.voff * 2u), o4 = (int)(cu.voff * 4u);
-  const int tok = (int)cu.tok_bytes;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    float f = 0.f;
-    uint16_t k = 0, b = 0, w = 0;
-    if (nvalid == CK || 4 * g + i < nvalid) {      // the first test is uniform: no lane predicate but in a partial chunk
-      f = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rf, o4, 2 * i * tok, 0));
-      k = __builtin_amdgcn_raw_buffer_load_b16(rk, o2, i * tok, 0);
-      b = __builtin_amdgcn_raw_buffer_load_b16(rb, o2, i * tok, 0);
-      w = __builtin_amdgcn_raw_buffer_load_b16(rw, o2, i * tok, 0);
-    }
-    p.f[i] = f;
-    p.k[i] = k; p.b[i] = b; p.w[i] = w;
-  }
-}
-
 __device__ __forceinline__ void step_back(Cursor& cu) {
   const size_t d = CK * cu.tok_bytes;
-  cu.ef -= 2 * d;
-  cu.k -= d; cu.b -= d; cu.w -= d;
   cu.gk -= d; cu.gb -= d; cu.gw -= d;
 }
 
@@ -361,8 +358,7 @@ __device__ __forceinline__ float ld_state_el(const void* p, int f32, size_t off)
 
 __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ slot, const SnapSlot* __restrict__ snapslot,
                                         const Wkv7Args& A, int64_t b, int64_t h, int nvalid, bool is_snap,
-                                        const Pre& pre, Pre& pre_next, const Cursor& cu, const Cursor& cu_next,
-                                        bool has_next) {
+                                        const Cursor& cu) {
   const int lane = C.lane, n = lane & 15, g = lane >> 4, q = C.q;
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
   // B operands of the token contractions: (a.Ee, r.E) of tokens 4g..4g+3 at this wave's keys
@@ -449,14 +445,22 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
     C.G[vt] = acc;
   }
   // per-token results: register i is token 4g+i, lanes n = 16 consecutive keys
-  float dk[4], db[4], z[4], cy[4];
+  float dk[4], db[4], z[4], cy[4], nej[4];
+  const float4 fr = slot->F[q][lane];
+  float fv[4] = {fr.x, fr.y, fr.z, fr.w};
+  if (nvalid != CK) {         // entries of tokens beyond the sequence hold nothing meaningful
+    rare_path();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) fv[i] = (4 * g + i < nvalid) ? fv[i] : 0.f;
+  }
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const float ei = slot->Einv[4 * g + i][16 * q + n];
     dk[i] = DK[i] * ei;
     db[i] = DB[i] * ei;
-    const float kk = bf16_to_f32(pre.k[i]), bb = bf16_to_f32(pre.b[i]);
-    z[i] = pre.f[i] - kk * dk[i] - bb * db[i];
+    const float kk = bf16_to_f32(slot->KBW[0][4 * g + i][16 * q + n]), bb = bf16_to_f32(slot->KBW[1][4 * g + i][16 * q + n]);
+    z[i] = fv[i] - kk * dk[i] - bb * db[i];
+    nej[i] = -__expf(bf16_to_f32(slot->KBW[2][4 * g + i][16 * q + n]));
   }
   // carry_t = reset_t ? 0 : carry_{t+1} + z_t, from token 15 down
   if (resets == 0) {
@@ -478,17 +482,8 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
   uint16_t ok[4], ob[4], ow[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const float nej = -__expf(bf16_to_f32(pre.w[i]));
-    ok[i] = f32_to_bf16(dk[i]); ob[i] = f32_to_bf16(db[i]); ow[i] = f32_to_bf16(cy[i] * nej);
+    ok[i] = f32_to_bf16(dk[i]); ob[i] = f32_to_bf16(db[i]); ow[i] = f32_to_bf16(cy[i] * nej[i]);
   }
-  // The next chunk's per-token scalars are requested after the last read of this chunk's (into a second set of
-  // registers: the caller alternates two sets, so nothing is copied) and before this chunk's stores.  Loads and
-  // stores share one in-order counter, a wait for a load also waits for every older store, and the compiler drains
-  // the counter completely whenever both kinds are in flight: in this order everything in flight at the next wait
-  // is a whole chunk old.  The barriers keep the scheduler from moving the loads up or the stores above them.
-  __builtin_amdgcn_sched_barrier(0);
-  if (has_next) prefetch(pre_next, cu_next, CK, g);
-  __builtin_amdgcn_sched_barrier(0);
   const rsrc_t rgk = make_rsrc(cu.gk), rgb = make_rsrc(cu.gb), rgw = make_rsrc(cu.gw);
   const int o2 = (int)(cu.voff * 2u), tokb = (int)cu.tok_bytes;
   auto put = [&](int i, bool full) {
@@ -542,34 +537,21 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_bwd_c_kernel(
     Cursor cu;
     cu.tok_bytes = (size_t)A.H * 64 * 2;
     const size_t el0 = (((size_t)b * A.T + (size_t)(nch - 1) * CK) * A.H + h) * 64;
-    cu.ef = reinterpret_cast<const char*>(A.e2) + el0 * 4;
-    cu.k = reinterpret_cast<const char*>(A.k) + el0 * 2;
-    cu.b = reinterpret_cast<const char*>(A.b) + el0 * 2;
-    cu.w = reinterpret_cast<const char*>(A.w) + el0 * 2;
     cu.gk = reinterpret_cast<char*>(A.gk) + el0 * 2;
     cu.gb = reinterpret_cast<char*>(A.gb) + el0 * 2;
     cu.gw = reinterpret_cast<char*>(A.gw) + el0 * 2;
     cu.voff = (uint32_t)((4 * g) * (int)A.H * 64 + 16 * wave + n);
     const int csnap = (L >= 1 && inject) ? (int)((L - 1) / CK) : -1;
     const int tail = (A.T % CK == 0) ? CK : (int)(A.T % CK);
-    Pre pre_a, pre_b;
-    if (nch > 0) prefetch(pre_a, cu, tail, g);
-    auto step = [&](int j, const Pre& pre, Pre& pre_next) -> bool {
+    for (int j = 0; j < nch; ++j) {
       const int c = nch - 1 - j;
       const int nvalid = (j == 0) ? tail : CK;
       const int si = j % RING;
-      Cursor nxt = cu;
-      step_back(nxt);
-      if (!wait_ready(sy, si, j + 1)) return false;
-      consume(C, &slots[si], snapslot, A, b, h, nvalid, c == csnap, pre, pre_next, cu, nxt, j + 1 < nch);
-      cu = nxt;
+      if (!wait_ready(sy, si, j + 1)) break;
+      consume(C, &slots[si], snapslot, A, b, h, nvalid, c == csnap, cu);
+      step_back(cu);
       // every LDS read of slot si has returned: its data went into the MFMAs and stores above
       if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
-      return true;
-    };
-    for (int j = 0; j < nch; j += 2) {      // two steps per turn: the prefetch registers alternate
-      if (!step(j, pre_a, pre_b)) break;
-      if (j + 1 < nch && !step(j + 1, pre_b, pre_a)) break;
     }
   } else {
     const int p = wave - NCONS;
@@ -599,6 +581,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_chunk_bwd_c_kernel(
       // the release orders this wave's LDS writes before the sequence number
       if (lane == 0) __hip_atomic_store(&sy->ready[si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
+    retire_loads(raw, ns_mine);
   }
   __syncthreads();
   if (head_broken(sy, A.status)) {

@@ -620,10 +620,12 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_fwd_kernel(Wkv7Args
   } else {
     const int p = pp;
     Raw raw;
-    uint32_t ns_mine = 0u;      // this lane's new_starts byte of the chunk loaded next: fetched a step ahead, like the operands
+    // this lane's new_starts byte of the chunk loaded next: fetched a step ahead, behind the operands (measured: 1.6 %
+    // faster here than in front of them, where the other sweeps have it)
+    uint32_t ns_mine = 0u;
     if (p < nch) {
-      ns_mine = chunk_flag_prefetch(A.ns, A.T, b, (int64_t)p * CK, lane);
       load_raw(raw, A, b, h, (int64_t)p * CK, lane);
+      ns_mine = chunk_flag_prefetch(A.ns, A.T, b, (int64_t)p * CK, lane);
     }
     for (int j = p; j < nch; j += NPROD) {
       const int64_t c0 = (int64_t)j * CK;
@@ -634,13 +636,14 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_fwd_kernel(Wkv7Args
       mask_raw(raw, F.nvalid, lane);
       produce(lane, raw, F, slot, snapslot, events_word(A.status));
       if (j + NPROD < nch) {
-        ns_mine = chunk_flag_prefetch(A.ns, A.T, b, c0 + (int64_t)NPROD * CK, lane);
         load_raw(raw, A, b, h, c0 + (int64_t)NPROD * CK, lane);
+        ns_mine = chunk_flag_prefetch(A.ns, A.T, b, c0 + (int64_t)NPROD * CK, lane);
       }
       if ((A.flags & FLAG_DROP_PUBLISH) && j + 1 == nch) break;
       // the release orders this wave's LDS writes before the sequence number
       if (lane == 0) __hip_atomic_store(&sy->ready[si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
+    retire_loads(raw, ns_mine);
   }
   __syncthreads();
   if (head_broken(sy, A.status)) {
