@@ -286,6 +286,28 @@ def bench_wkv7(torch, ops, args):
                           "hbm_frac": b32 / (k32 * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": b32,
                           "mfma_frac": None if args.seq else fp32_mfma_flops(tokens) / (k32 * 1e-3) / 1e12 / 157.3,
                           "kernel": "sequential fp32 VALU" if args.seq else "chunked, v_mfma_f32_16x16x4_f32 (fp32 operands)"}
+        if not args.no_bwd:
+            # forward (keeping the fp32 residual sa) + the three backward sweeps, all with fp32 I/O
+            dy32 = x["dy"].float()
+
+            def fwd_bwd32():
+                new_s, y, sa = ops.wkv7_fwd(x32["r"], x32["w"], x32["k"], x32["v"], x32["a"], x32["b"], x32["s"],
+                                            x32["length"], x32["new_starts"], compat=True, want_sa=True, force_seq=args.seq)
+                return ops.wkv7_bwd(x32["r"], x32["w"], x32["k"], x32["v"], x32["a"], x32["b"], x32["s"], x32["length"],
+                                    x32["new_starts"], dy32, sa, None, compat=True, force_seq=args.seq)
+            n5 = max(2, args.steps // 10)
+            wall5, _ = time_region(torch, fwd_bwd32, n5, 1)
+            ms5 = 1e3 * wall5 / n5
+            fb32 = 20 * tokens * H * N * 4 + 4 * B * H * N * N * 4
+            out["fp32_io"]["fwd_bwd_ms"] = ms5
+            out["fp32_io"]["fwd_bwd_tokens_per_s"] = tokens / (ms5 * 1e-3)
+            out["fp32_io"]["fwd_bwd_hbm_frac"] = fb32 / (ms5 * 1e-3) / 1e9 / HBM_PEAK_GBS
+            # matrix instructions per (chunk, head): forward and sweep A 4 x 80 (consumers) + 96 (producer) each,
+            # sweeps B and C 4 x 80 + 64 each; 2048 flop per instruction
+            if not args.seq:
+                mf = (2 * 416 + 2 * 384) * 2048 * (tokens // 16) * H
+                out["fp32_io"]["fwd_bwd_mfma_frac"] = mf / (ms5 * 1e-3) / 1e12 / 157.3
+            del dy32
         del x32
     if not args.no_placement and not args.seq:
         # The same two measurements with the seven input arrays copied to addresses 0, 128, ..., 768 bytes past a 1 KiB

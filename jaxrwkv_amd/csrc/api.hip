@@ -254,12 +254,16 @@ int hiprwkv_wkv7_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64
   A.e3 = reinterpret_cast<float*>(at_phase(reinterpret_cast<char*>(A.e2) + one, r, 7));
   // Three sweeps: A (reverse) -> gv, dsa, gs; B (forward) -> gr, ga, e2, e3 (the chunked B: their sum shifted by a
   // token, in e2); C (reverse) -> gk, gb, gw.
-  // bf16 I/O runs all three on the chunked MFMA kernels.
-  const bool chunked = io_dtype == HIPRWKV_BF16 && !(flags & HIPRWKV_FORCE_SEQ);
+  // All three run on the chunked matrix-core kernels (bf16 pairs for bf16 I/O, fp32 operands for fp32 I/O);
+  // HIPRWKV_FORCE_SEQ selects the sequential kernels.
+  const bool chunked = !(flags & HIPRWKV_FORCE_SEQ);
+  const bool f32 = A.io_f32 != 0;
   hipStream_t st = static_cast<hipStream_t>(stream);
-  hipError_t e = chunked ? launch_wkv7_chunk_bwd_a(A, st) : launch_wkv7_seq_bwd_a(A, st);
-  if (e == hipSuccess) e = chunked ? launch_wkv7_chunk_bwd_b(A, st) : launch_wkv7_seq_bwd_b(A, st);
-  if (e == hipSuccess) e = chunked ? launch_wkv7_chunk_bwd_c(A, st) : launch_wkv7_seq_bwd_c(A, st);
+  hipError_t e = !chunked ? launch_wkv7_seq_bwd_a(A, st) : f32 ? launch_wkv7_chunk_bwd_a_f32(A, st) : launch_wkv7_chunk_bwd_a(A, st);
+  if (e == hipSuccess)
+    e = !chunked ? launch_wkv7_seq_bwd_b(A, st) : f32 ? launch_wkv7_chunk_bwd_b_f32(A, st) : launch_wkv7_chunk_bwd_b(A, st);
+  if (e == hipSuccess)
+    e = !chunked ? launch_wkv7_seq_bwd_c(A, st) : f32 ? launch_wkv7_chunk_bwd_c_f32(A, st) : launch_wkv7_chunk_bwd_c(A, st);
   if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "wkv7_bwd: %s", hipGetErrorString(e));
   return HIPRWKV_OK;
 }

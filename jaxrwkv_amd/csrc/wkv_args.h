@@ -93,6 +93,9 @@ inline hipError_t allow_dynamic_lds(LdsAttrOnce& once, const void* kernel, size_
 hipError_t launch_wkv7_seq_fwd(const Wkv7Args& A, hipStream_t stream);
 hipError_t launch_wkv7_chunk_fwd(const Wkv7Args& A, hipStream_t stream);
 hipError_t launch_wkv7_chunk_fwd_f32(const Wkv7Args& A, hipStream_t stream);
+hipError_t launch_wkv7_chunk_bwd_a_f32(const Wkv7Args& A, hipStream_t stream);
+hipError_t launch_wkv7_chunk_bwd_b_f32(const Wkv7Args& A, hipStream_t stream);
+hipError_t launch_wkv7_chunk_bwd_c_f32(const Wkv7Args& A, hipStream_t stream);
 hipError_t launch_wkv7_small_t_fwd(const Wkv7Args& A, hipStream_t stream);
 hipError_t launch_wkv6_small_t_fwd(const Wkv6Args& A, hipStream_t stream);
 hipError_t launch_wkv7_chunk_bwd_a(const Wkv7Args& A, hipStream_t stream);
