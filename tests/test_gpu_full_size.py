@@ -46,6 +46,28 @@ def test_wkv7_forward_and_backward_chunked_equals_sequential_at_the_headline_sha
         assert rel_rms(c, q) < tol[n_], (n_, rel_rms(c, q))
 
 
+def test_wkv7_fp32_forward_and_backward_chunked_equals_sequential_at_the_headline_shape():
+    """fp32 I/O at B=8 T=4096 H=32: the chunked kernels on fp32 matrix instructions against the sequential fp32 kernels,
+    forward and all seven cotangents.  Both compute in fp32 throughout, so they agree to a few 1e-6 in relative rms
+    (1e-4 for the decay gradient, a running sum over up to 4096 tokens of terms that cancel)."""
+    from jaxrwkv_amd import ops
+    x = wkv7_full(seed=6)
+    args = tuple(x[n].float() for n in "rwkvab") + (x["s"], x["length"], x["ns"])
+    dy, ds = x["dy"].float(), torch.randn_like(x["s"])
+    out = {}
+    for fs in (False, True):
+        new_s, y, sa = ops.wkv7_fwd(*args, compat=True, want_sa=True, force_seq=fs)
+        g = ops.wkv7_bwd(*args, dy, sa, ds, compat=True, force_seq=fs)
+        out[fs] = (new_s, y, sa) + tuple(g)
+    torch.cuda.synchronize()
+    names = ("new_s", "y", "sa", "gr", "gw", "gk", "gv", "ga", "gb", "gs")
+    for n_, c, q in zip(names, out[False], out[True]):
+        assert c.dtype == torch.float32 and torch.isfinite(c).all(), n_
+        assert rel_rms(c, q) < (1e-4 if n_ == "gw" else 1e-5), (n_, rel_rms(c, q))
+    # the cotangents vanish exactly where the forward is cut: dsa-driven ga at every reset token
+    assert torch.count_nonzero(out[False][7][x["ns"]]) == 0
+
+
 def test_wkv7_split_call_with_carried_state_equals_single_call_at_the_headline_shape():
     from jaxrwkv_amd import ops
     x = wkv7_full(seed=1)

@@ -60,8 +60,8 @@ def test_wkv7(case):
 
 @pytest.mark.parametrize("case", CASES, ids=lambda c: "B{B}-T{T}-H{H}-p{p}-c{compat:d}-f{frac}".format(**c))
 def test_wkv7_fp32(case):
-    """fp32 I/O: the chunked kernel on fp32 matrix instructions and the sequential kernel, both at the fp32 bar
-    (rtol 1e-4, atol 1e-5), with exact zeros at the reset positions."""
+    """fp32 I/O: the chunked kernels on fp32 matrix instructions and the sequential kernels, forward and backward, both
+    at the fp32 bar (rtol 1e-4, atol 1e-5; cotangents in units of their rms), with exact zeros at the reset positions."""
     from tests import test_gpu_wkv7 as t7
     B, T, H, compat = case["B"], case["T"], case["H"], case["compat"]
     x = wkv7_inputs(B, T, H, 64, seed=case["seed"], p_reset=case["p"], min_len_frac=case["frac"])
@@ -75,6 +75,12 @@ def test_wkv7_fp32(case):
         assert_close("new_s", new_s, ref_s)
         assert_close("sa", sa, ref_sa)
         assert np.all(sa[x["new_starts"]] == 0.0)
+    ref = o7.wkv7_bwd(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], x["length"], x["new_starts"], x["dy"],
+                      x["ds"], compat=compat)
+    for force_seq in (False, True):      # the three sweeps on fp32 matrix instructions, and the sequential ones
+        got = t7.run_bwd(x, torch.float32, compat, force_seq)
+        for n, g, rf in zip("rwkvabs", got, ref):
+            assert_close("g" + n, g, rf, atol=t7.GRAD_ATOL[n], scale_atol=True)
 
 
 @pytest.mark.parametrize("case", CASES, ids=lambda c: "B{B}-T{T}-H{H}-p{p}-c{compat:d}-f{frac}".format(**c))

@@ -26,11 +26,12 @@ def run_fwd(x, dtype, compat, state_dtype=torch.float32, force_seq=False):
     return host(new_s), host(y), host(sa)
 
 
-def run_bwd(x, dtype, compat):
+def run_bwd(x, dtype, compat, force_seq=False):
     from jaxrwkv_amd import ops
     t = {n: dev(x[n], dtype).requires_grad_() for n in ("r", "w", "k", "v", "a", "b")}
     s = dev(x["s"]).requires_grad_()
-    new_s, y = ops.wkv7(t["r"], t["w"], t["k"], t["v"], t["a"], t["b"], s, dev(x["length"]), dev(x["new_starts"]), compat=compat)
+    new_s, y = ops.wkv7(t["r"], t["w"], t["k"], t["v"], t["a"], t["b"], s, dev(x["length"]), dev(x["new_starts"]), compat=compat,
+                        force_seq=force_seq)
     loss = (y.float() * dev(x["dy"])).sum() + (new_s * dev(x["ds"])).sum()
     loss.backward()
     torch.cuda.synchronize()
@@ -91,26 +92,64 @@ def test_length_zero_and_none():
     assert_close("new_s", host(new_s), ref_s)
 
 
+# fp32 I/O runs on the chunked kernels with fp32 matrix operands by default and on the sequential kernels with
+# force_seq: both are held to the same bar against the float64 oracle.
+@pytest.mark.parametrize("force_seq", [False, True], ids=["chunked", "seq"])
 @pytest.mark.parametrize("compat", [True, False])
 @pytest.mark.parametrize("B,T,H,seed", [(2, 48, 2, 21), (1, 97, 3, 22)])
-def test_fp32_backward(B, T, H, seed, compat):
+def test_fp32_backward(B, T, H, seed, compat, force_seq):
     x = wkv7_inputs(B, T, H, 64, seed=seed, p_reset=0.04, min_len_frac=0.4)
     x["length"][0] = T // 2
     x["new_starts"][0, T // 2] = True
     ref = o7.wkv7_bwd(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], x["length"], x["new_starts"], x["dy"], x["ds"], compat=compat)
-    got = run_bwd(x, torch.float32, compat)
+    got = run_bwd(x, torch.float32, compat, force_seq)
     for n, g, rf in zip("rwkvabs", got, ref):
         assert_close("g" + n, g, rf, atol=GRAD_ATOL[n], scale_atol=True)
 
 
-def test_backward_length_zero():
+@pytest.mark.parametrize("force_seq", [False, True], ids=["chunked", "seq"])
+def test_backward_length_zero(force_seq):
     x = wkv7_inputs(2, 12, 1, 64, seed=23, p_reset=0.1)
     x["length"][:] = 0
     for compat in (True, False):
         ref = o7.wkv7_bwd(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], x["length"], x["new_starts"], x["dy"], x["ds"], compat=compat)
-        got = run_bwd(x, torch.float32, compat)
+        got = run_bwd(x, torch.float32, compat, force_seq)
         for n, g, rf in zip("rwkvabs", got, ref):
             assert_close("g" + n, g, rf, atol=GRAD_ATOL[n], scale_atol=True)
+
+
+@pytest.mark.parametrize("B,T,H,p,seed", [(1, 640, 2, 0.0, 31), (1, 1100, 1, 0.004, 32), (2, 333, 2, 0.02, 33), (1, 2048, 1, 0.0, 35)])
+def test_fp32_backward_long(B, T, H, p, seed):
+    """Hundreds of chunks: the carried cotangent, the running sum of the decay gradient and the records handed from the
+    forward sweep to the last one, all in fp32 against the float64 oracle; the length of one sequence ends inside a
+    chunk, with a reset right after it.  The decay gradient at token t is a sum over every later token of the segment
+    of terms that cancel, each an fp32 result: its error grows with the distance to the end.  Measured at 640-2048
+    tokens without resets: 2.0-2.55 times the bound of the short cases for these kernels and 1.8-2.05 times for the
+    sequential ones (a compensated carry changes nothing: the terms' own rounding is what adds up), so gw is held to
+    2e-4 of its rms here and the other cotangents to the bound of the short cases."""
+    x = wkv7_inputs(B, T, H, 64, seed=seed, p_reset=p, min_len_frac=0.6)
+    x["length"][0] = T - 37
+    x["new_starts"][0, T - 37] = True
+    ref = o7.wkv7_bwd(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], x["length"], x["new_starts"], x["dy"], x["ds"], compat=True)
+    got = run_bwd(x, torch.float32, True)
+    for n, g, rf in zip("rwkvabs", got, ref):
+        assert_close("g" + n, g, rf, atol=2e-4 if n == "w" else GRAD_ATOL[n], scale_atol=True)
+
+
+def test_fp32_backward_with_bf16_state():
+    """fp32 token tensors with a bf16 state and state cotangent (the state dtype is independent of the I/O dtype)."""
+    from jaxrwkv_amd import ops
+    x = wkv7_inputs(2, 50, 2, 64, seed=34, p_reset=0.03, min_len_frac=0.5)
+    x["s"], x["ds"] = bf16_round(x["s"]), bf16_round(x["ds"])
+    ref = o7.wkv7_bwd(x["r"], x["w"], x["k"], x["v"], x["a"], x["b"], x["s"], x["length"], x["new_starts"], x["dy"], x["ds"], compat=True)
+    t = [dev(x[n], torch.float32) for n in ("r", "w", "k", "v", "a", "b")]
+    s, ln, ns = dev(x["s"], torch.bfloat16), dev(x["length"]), dev(x["new_starts"])
+    _, _, sa = ops.wkv7_fwd(*t, s, ln, ns, compat=True, want_sa=True, small_t=False)
+    got = ops.wkv7_bwd(*t, s, ln, ns, dev(x["dy"], torch.float32), sa, dev(x["ds"], torch.bfloat16), compat=True)
+    torch.cuda.synchronize()
+    for n, g, rf in zip("rwkvab", got[:6], ref[:6]):
+        assert_close("g" + n, host(g), rf, atol=GRAD_ATOL[n], scale_atol=True)
+    assert_close("gs", host(got[6].float()), ref[6], rtol=2.0 ** -7, atol=1e-5)
 
 
 def test_bf16_io_against_float64_oracle():
