@@ -137,7 +137,10 @@ size_t hiprwkv_wkv7_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t
 /* Replaces ffi target "wkv7-bwd-{fp32,bf16}": operands w,r,k,v,a,b,s,length,new_starts,
  * gy,s_restore,sa_restore,gs_out -> gw,gr,gk,gv,ga,gb,gs  (rwkv7.py:406-408).
  * Unlike the reference's native op it honours new_starts, takes the cotangent of the
- * returned state (gs_out, may be NULL = 0) and returns the one of the input state. */
+ * returned state (gs_out, may be NULL = 0) and returns the one of the input state.
+ * Three sweeps over the sequence on the matrix cores: bf16 hi+lo operand pairs beside bf16
+ * I/O, fp32 operands (no rounding below fp32) beside fp32 I/O; HIPRWKV_FORCE_SEQ runs the
+ * sequential fp32 sweeps instead. */
 int hiprwkv_wkv7_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype,
                      int64_t B, int64_t T, int64_t H, int64_t N,
                      const void* w, const void* r, const void* k, const void* v,
