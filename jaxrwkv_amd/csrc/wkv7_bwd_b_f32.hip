@@ -31,7 +31,7 @@ namespace {
 using namespace chunk;
 
 constexpr int NPROD = 4;          // producer waves; producer p owns chunks p, p + NPROD, ...
-constexpr int RING = 3;           // slots in flight (a slot is 43 KB)
+constexpr int RING = 4;           // slots in flight (a slot is 35 KB); with three, one of the four producers always idles: +10 %
 constexpr float LN2 = 0.69314718055994530942f;
 constexpr float GRID_MAGIC = 192.f;   // (x + 192) - 192 rounds |x| < 64 to a multiple of 2^-16
 constexpr int RF = 68;            // row stride (floats) of the [token][64] LDS arrays: rows 4 apart fall 16 banks apart
@@ -47,8 +47,6 @@ struct __attribute__((aligned(16))) Slot {
   float V[CK][RF];             // v rows, masked likewise
   float BH[CK][RF];            // b_s/E_s rows [token][key]
   float KH[CK][RF];            // k_s/E_s rows
-  float R[CK][RF];             // r and a rows as loaded
-  float Aa[CK][RF];
   float E[CK + 1][RF];         // row t+1 = E_t per key, row 0 = 1
   f32x4_t Nys[64], Nyv[64];    // sa_s.dy_t, v_s.dy_t (s <= t), accumulator layout [row s][column t], lane-indexed
   f32x4_t Nss[64], Nsv[64];    // sa_s.dsa_t, v_s.dsa_t (s < t)
@@ -68,7 +66,7 @@ struct __attribute__((aligned(16))) SnapSlot {   // update operands with the tok
 // Lane (t = lane%16, g = lane/16) owns token t and, of every 64-vector, the elements 16j + 4g + i (j, i = 0..3): one
 // 16-byte load per j, and element (j, i) is this lane's k-slot of the Gram instruction (j, i) both as A and as B operand.
 struct Raw {
-  float4 w[4], k[4], b[4], r[4], a[4], v[4], dy[4], sa[4], dsa[4];
+  float4 w[4], k[4], b[4], v[4], dy[4], sa[4], dsa[4];
 };
 
 __device__ __forceinline__ void load_raw(Raw& x, const Wkv7Args& A, int64_t b, int64_t h, int64_t c0, int lane) {
@@ -79,7 +77,7 @@ __device__ __forceinline__ void load_raw(Raw& x, const Wkv7Args& A, int64_t b, i
 #pragma unroll
     for (int j = 0; j < 4; ++j) o[j] = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p) + off + 16 * j);
   };
-  ld(A.w, x.w); ld(A.k, x.k); ld(A.b, x.b); ld(A.r, x.r); ld(A.a, x.a);
+  ld(A.w, x.w); ld(A.k, x.k); ld(A.b, x.b);
   ld(A.v, x.v); ld(A.gy, x.dy); ld(A.sa_in, x.sa); ld(A.dsa, x.dsa);
 }
 __device__ __forceinline__ void mask_raw(Raw& x, int nvalid, int lane) {
@@ -88,7 +86,7 @@ __device__ __forceinline__ void mask_raw(Raw& x, int nvalid, int lane) {
     if ((lane & 15) >= nvalid) {
       const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) x.w[j] = x.k[j] = x.b[j] = x.r[j] = x.a[j] = x.v[j] = x.dy[j] = x.sa[j] = x.dsa[j] = z;
+      for (int j = 0; j < 4; ++j) x.w[j] = x.k[j] = x.b[j] = x.v[j] = x.dy[j] = x.sa[j] = x.dsa[j] = z;
     }
   }
 }
@@ -135,7 +133,7 @@ __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags
   f32x4_t Nys = zero4, Nyv = zero4, Nss = zero4, Nsv = zero4;
 #pragma unroll
   for (int hf = 0; hf < 2; ++hf) {
-    // ================= keys of this half: decay scan, b/E, k/E, E rows, r and a rows
+    // ================= keys of this half: decay scan, b/E, k/E, E rows
     {
       // Decay scan over the 16 tokens (lanes of one DPP row), log2 domain: every step is split into a part on a 2^-16
       // grid, whose running sums are exact, and a remainder below 2^-17, summed separately.
@@ -210,11 +208,6 @@ __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags
       }
       put2(slot->BH[t], hf, g, fbh, true);
       put2(slot->KH[t], hf, g, fkh, true);
-      float fr[8], fa[8];
-      unpack2(x.r[2 * hf], x.r[2 * hf + 1], fr);
-      unpack2(x.a[2 * hf], x.a[2 * hf + 1], fa);
-      put2(slot->R[t], hf, g, fr, true);
-      put2(slot->Aa[t], hf, g, fa, true);
     }
     // ================= values of this half: sa, v, dy and dsa rows, partial Gram sums
     {
@@ -294,8 +287,26 @@ __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags
 struct Consumer {
   f32x4_t S[4];
   float pend;          // lanes g = 3: r.dr of the previous chunk's last token, whose workspace entry is still open
+  // r and a of this lane's four (token, key) pairs of the chunk handled next: fetched from memory by the consumer
+  // itself, one chunk ahead, instead of passing through the LDS slot (8.5 KB per slot: the difference between a ring of
+  // three and one of four)
+  float rr[4], aa[4];
   int q, lane;
 };
+
+// r and a at (tokens c0 + 4g .. + 3, key 16q + n); tokens beyond the sequence read the last one (their results are
+// never stored)
+__device__ __forceinline__ void fetch_ra(Consumer& C, const Wkv7Args& A, int64_t b, int64_t h, int64_t c0) {
+  const int n = C.lane & 15, g = C.lane >> 4;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int64_t tok = c0 + 4 * g + i;
+    tok = tok < A.T ? tok : A.T - 1;
+    const size_t el = (((size_t)b * A.T + tok) * A.H + h) * 64 + 16 * C.q + n;
+    C.rr[i] = reinterpret_cast<const float*>(A.r)[el];
+    C.aa[i] = reinterpret_cast<const float*>(A.a)[el];
+  }
+}
 
 struct OutCursor {
   float *gr, *ga;      // outputs at (b, c0, h, 0)
@@ -313,9 +324,11 @@ __device__ __forceinline__ float ld_state_el(const void* p, int f32, size_t off)
 
 __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ slot, const SnapSlot* __restrict__ snapslot,
                                         const Wkv7Args& A, int64_t b, int64_t h, int nvalid, bool is_snap, bool first,
-                                        OutCursor& oc) {
+                                        int64_t next_c0, OutCursor& oc) {
   const int lane = C.lane, n = lane & 15, g = lane >> 4, q = C.q;
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
+  const float rr[4] = {C.rr[0], C.rr[1], C.rr[2], C.rr[3]}, aa[4] = {C.aa[0], C.aa[1], C.aa[2], C.aa[3]};
+  if (next_c0 >= 0) fetch_ra(C, A, b, h, next_c0);
   // B operands of the token contractions: (b/E, k/E) of tokens 4g..4g+3 at this wave's keys
   float tb[4], tk[4];
 #pragma unroll
@@ -401,12 +414,10 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int tok = 4 * g + i;
-    const float rr = slot->R[tok][16 * q + n];
-    const float aa = slot->Aa[tok][16 * q + n];
     odr[i] = DR[i] * e[i + 1];
     oda[i] = DA[i] * e[i];
-    e2[i] = aa * oda[i];
-    e3[i] = fmaf(rr, odr[i], tok == snap_tok ? inj : 0.f);
+    e2[i] = aa[i] * oda[i];
+    e3[i] = fmaf(rr[i], odr[i], tok == snap_tok ? inj : 0.f);
   }
   if (!full) {
     rare_path();
@@ -493,11 +504,12 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_bwd_b_f32_kernel(Wk
     oc.ef = A.e2 + f_record(b, h, A.H, nch, 0, wave);
     oc.voff = (uint32_t)((4 * g) * (int)A.H * 64 + 16 * wave + n);
     const int csnap = (L >= 1 && inject) ? (int)((L - 1) / CK) : -1;
+    if (nch > 0) fetch_ra(C, A, b, h, 0);
     for (int c = 0; c < nch; ++c) {
       const int nvalid = (c + 1 < nch || A.T % CK == 0) ? CK : (int)(A.T % CK);
       const int si = c % RING;
       if (!wait_ready(sy, si, c + 1)) break;
-      consume(C, &slots[si], snapslot, A, b, h, nvalid, c == csnap, c == 0, oc);
+      consume(C, &slots[si], snapslot, A, b, h, nvalid, c == csnap, c == 0, c + 1 < nch ? (int64_t)(c + 1) * CK : -1, oc);
       // every LDS read of slot si has returned: its data went into the matrix instructions and stores above
       if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], c + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }

@@ -24,7 +24,7 @@ namespace {
 using namespace chunk;
 
 constexpr int NPROD = 4;          // producer waves; producer p owns steps p, p + NPROD, ...
-constexpr int RING = 3;           // slots in flight (a slot is 47 KB)
+constexpr int RING = 4;           // slots in flight (a slot is 35 KB); with three, one of the four producers always idles
 constexpr float LN2 = 0.69314718055994530942f;
 constexpr float GRID_MAGIC = 192.f;   // (x + 192) - 192 rounds |x| < 64 to a multiple of 2^-16
 constexpr int RF = 68;            // row stride (floats) of the [token][64] LDS arrays: rows 4 apart fall 16 banks apart
@@ -44,9 +44,6 @@ struct __attribute__((aligned(16))) Slot {
   float AT[CK][RF];            // a_s.E_{s-1} rows [token][key]
   float QT[CK][RF];            // r_s.E_s rows
   float Einv[CK][RF];          // 1/E_t per key
-  float K[CK][RF];             // k and b rows as loaded
-  float Bb[CK][RF];
-  float NEJ[CK][RF];           // -exp(w) rows
   f32x4_t Nsv[64], Nyv[64];    // dsa_s.v_t (s > t), dy_s.v_t (s >= t), accumulator layout [row s][column t], lane-indexed
   f32x4_t Nss[64], Nys[64];    // dsa_s.sa_t (s > t), dy_s.sa_t (s >= t)
   float gamma[64];             // E at the chunk end
@@ -65,7 +62,7 @@ struct __attribute__((aligned(16))) SnapSlot {   // row operands masked to the t
 // Lane (t = lane%16, g = lane/16) owns token t and, of every 64-vector, the elements 16j + 4g + i (j, i = 0..3): one
 // 16-byte load per j, and element (j, i) is this lane's k-slot of the Gram instruction (j, i) both as A and as B operand.
 struct Raw {
-  float4 w[4], r[4], a[4], k[4], b[4], v[4], dy[4], sa[4], dsa[4];
+  float4 w[4], r[4], a[4], v[4], dy[4], sa[4], dsa[4];
 };
 
 __device__ __forceinline__ void load_raw(Raw& x, const Wkv7Args& A, int64_t b, int64_t h, int64_t c0, int lane) {
@@ -76,7 +73,7 @@ __device__ __forceinline__ void load_raw(Raw& x, const Wkv7Args& A, int64_t b, i
 #pragma unroll
     for (int j = 0; j < 4; ++j) o[j] = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(p) + off + 16 * j);
   };
-  ld(A.w, x.w); ld(A.r, x.r); ld(A.a, x.a); ld(A.k, x.k); ld(A.b, x.b);
+  ld(A.w, x.w); ld(A.r, x.r); ld(A.a, x.a);
   ld(A.v, x.v); ld(A.gy, x.dy); ld(A.sa_in, x.sa); ld(A.dsa, x.dsa);
 }
 __device__ __forceinline__ void mask_raw(Raw& x, int nvalid, int lane) {
@@ -85,7 +82,7 @@ __device__ __forceinline__ void mask_raw(Raw& x, int nvalid, int lane) {
     if ((lane & 15) >= nvalid) {
       const float4 z = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) x.w[j] = x.r[j] = x.a[j] = x.k[j] = x.b[j] = x.v[j] = x.dy[j] = x.sa[j] = x.dsa[j] = z;
+      for (int j = 0; j < 4; ++j) x.w[j] = x.r[j] = x.a[j] = x.v[j] = x.dy[j] = x.sa[j] = x.dsa[j] = z;
     }
   }
 }
@@ -132,9 +129,8 @@ __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags
   f32x4_t Nsv = zero4, Nyv = zero4, Nss = zero4, Nys = zero4;
 #pragma unroll
   for (int hf = 0; hf < 2; ++hf) {
-    // ================= keys of this half: decay scan, a.E_{t-1}, r.E_t, 1/E rows, k, b and -exp(w) rows
+    // ================= keys of this half: decay scan, a.E_{t-1}, r.E_t, 1/E rows
     {
-      float nej[8];
       // Decay scan over the 16 tokens (lanes of one DPP row), log2 domain: every step is split into a part on a 2^-16
       // grid, whose running sums are exact, and a remainder below 2^-17, summed separately.
       float E[8], El[8];
@@ -142,10 +138,7 @@ __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags
         float fw[8];
         unpack2(x.w[2 * hf], x.w[2 * hf + 1], fw);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) {
-          nej[e] = -exp2_fast(fw[e] * LOG2E);           // -exp(w): the factor between the log-decay gradient and gw
-          fw[e] = fmaxf(nej[e] * LOG2E, MIN_STEP_L2);
-        }
+        for (int e = 0; e < 8; ++e) fw[e] = fmaxf(-exp2_fast(fw[e] * LOG2E) * LOG2E, MIN_STEP_L2);
         if (F.nvalid != CK) {
           rare_path();
 #pragma unroll
@@ -210,12 +203,6 @@ __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags
       }
       put2(slot->AT[t], hf, g, fat, true);
       put2(slot->QT[t], hf, g, fqt, true);
-      float fk[8], fb[8];
-      unpack2(x.k[2 * hf], x.k[2 * hf + 1], fk);
-      unpack2(x.b[2 * hf], x.b[2 * hf + 1], fb);
-      put2(slot->K[t], hf, g, fk, true);
-      put2(slot->Bb[t], hf, g, fb, true);
-      put2(slot->NEJ[t], hf, g, nej, true);
     }
     // ================= values of this half: v, sa, dy and dsa rows, partial Gram sums
     {
@@ -295,8 +282,27 @@ struct Consumer {
   f32x4_t G[4];
   float carry;         // running sum of the decay-gradient recursion, per key (same in the four lanes of a key)
   float4 f;            // this wave's record entry of the chunk handled next (requested one chunk ahead)
+  // k, b and w of this lane's four (token, key) pairs of the chunk handled next: fetched from memory by the consumer
+  // itself, one chunk ahead, instead of passing through the LDS slot (13 KB per slot: the difference between a ring of
+  // three and one of four)
+  float kk[4], bb[4], ww[4];
   int q, lane;
 };
+
+// k, b, w at (tokens c0 + 4g .. + 3, key 16q + n); tokens beyond the sequence read the last one (their results are
+// never stored)
+__device__ __forceinline__ void fetch_kbw(Consumer& C, const Wkv7Args& A, int64_t b, int64_t h, int64_t c0) {
+  const int n = C.lane & 15, g = C.lane >> 4;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int64_t tok = c0 + 4 * g + i;
+    tok = tok < A.T ? tok : A.T - 1;
+    const size_t el = (((size_t)b * A.T + tok) * A.H + h) * 64 + 16 * C.q + n;
+    C.kk[i] = reinterpret_cast<const float*>(A.k)[el];
+    C.bb[i] = reinterpret_cast<const float*>(A.b)[el];
+    C.ww[i] = reinterpret_cast<const float*>(A.w)[el];
+  }
+}
 
 struct Cursor {
   float *gk, *gb, *gw;         // outputs at (b, c0, h, 0)
@@ -314,14 +320,17 @@ __device__ __forceinline__ float ld_state_el(const void* p, int f32, size_t off)
 
 __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ slot, const SnapSlot* __restrict__ snapslot,
                                         const Wkv7Args& A, int64_t b, int64_t h, int nvalid, bool is_snap, bool last,
-                                        Cursor& cu) {
+                                        int64_t next_c0, Cursor& cu) {
   const int lane = C.lane, n = lane & 15, g = lane >> 4, q = C.q;
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
-  // this chunk's record entry was requested a chunk ago; request the next one
+  // this chunk's record entry and per-token scalars were requested a chunk ago; request the next ones
   const float4 fr = C.f;
+  const float kk[4] = {C.kk[0], C.kk[1], C.kk[2], C.kk[3]}, bb[4] = {C.bb[0], C.bb[1], C.bb[2], C.bb[3]};
+  const float ww[4] = {C.ww[0], C.ww[1], C.ww[2], C.ww[3]};
   if (!last) {
     cu.rec -= NCONS * (F_REC / 4);
     C.f = *cu.rec;
+    fetch_kbw(C, A, b, h, next_c0);
   }
   // B operands of the token contractions: (a.E_{s-1}, r.E_s) of tokens 4g..4g+3 at this wave's keys
   float ta[4], tq[4];
@@ -412,9 +421,8 @@ __device__ __forceinline__ void consume(Consumer& C, const Slot* __restrict__ sl
     const float ei = slot->Einv[4 * g + i][16 * q + n];
     dk[i] = DK[i] * ei;
     db[i] = DB[i] * ei;
-    const float kk = slot->K[4 * g + i][16 * q + n], bb = slot->Bb[4 * g + i][16 * q + n];
-    z[i] = fv[i] - kk * dk[i] - bb * db[i];
-    nej[i] = slot->NEJ[4 * g + i][16 * q + n];
+    z[i] = fv[i] - kk[i] * dk[i] - bb[i] * db[i];
+    nej[i] = -exp2_fast(ww[i] * LOG2E);      // -exp(w): the factor between the log-decay gradient and gw
   }
   // carry_t = reset_t ? 0 : carry_{t+1} + z_t, from token 15 down
   if (resets == 0) {
@@ -499,7 +507,10 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_bwd_c_f32_kernel(Wk
     cu.rec = reinterpret_cast<const float4*>(A.e2 + f_record(b, h, A.H, nch, nch - 1, wave)) + lane;
     cu.voff = (uint32_t)((4 * g) * (int)A.H * 64 + 16 * wave + n);
     C.f = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (nch > 0) C.f = *cu.rec;
+    if (nch > 0) {
+      C.f = *cu.rec;
+      fetch_kbw(C, A, b, h, (int64_t)(nch - 1) * CK);
+    }
     const int csnap = (L >= 1 && inject) ? (int)((L - 1) / CK) : -1;
     const int tail = (A.T % CK == 0) ? CK : (int)(A.T % CK);
     for (int j = 0; j < nch; ++j) {
@@ -507,7 +518,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_bwd_c_f32_kernel(Wk
       const int nvalid = (j == 0) ? tail : CK;
       const int si = j % RING;
       if (!wait_ready(sy, si, j + 1)) break;
-      consume(C, &slots[si], snapslot, A, b, h, nvalid, c == csnap, j + 1 == nch, cu);
+      consume(C, &slots[si], snapslot, A, b, h, nvalid, c == csnap, j + 1 == nch, (int64_t)(c - 1) * CK, cu);
       // every LDS read of slot si has returned: its data went into the matrix instructions and stores above
       if (lane == 0) __hip_atomic_store(&sy->consumed[wave][si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
