@@ -399,6 +399,17 @@ def bench_wkv6(torch, ops, args):
         fb_bytes = 14 * tokens * H * N * 2 + 4 * b6 * H * N * N * 4
         out["fwd_bwd"] = {"tokens_per_s": tokens / (ms2 * 1e-3), "ms_per_step": ms2,
                           "hbm_frac": fb_bytes / (ms2 * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": fb_bytes}
+    if not args.no_fp32:
+        # the same shape with fp32 r/k/v/w/u/y: the chunked forward on fp32 matrix instructions, and the sequential
+        # kernel it replaces for fp32 I/O
+        r32, k32, v32, w32, u32 = (t.float() for t in (r, k, v, w, u))
+        n3 = max(2, args.steps // 4)
+        _, kc = time_region(torch, lambda: ops.wkv6_fwd(r32, k32, v32, w32, u32, s, None, ns, compat=True), n3, 2)
+        _, ks = time_region(torch, lambda: ops.wkv6_fwd(r32, k32, v32, w32, u32, s, None, ns, compat=True, force_seq=True), n3, 2)
+        b32 = 5 * tokens * H * N * 4 + 2 * b6 * H * N * N * 4 + b6 * t6
+        out["fp32_io"] = {"kernel_ms": kc, "tokens_per_s": tokens / (kc * 1e-3),
+                          "hbm_frac": b32 / (kc * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": b32,
+                          "sequential_kernel_ms": ks, "kernel": "chunked, v_mfma_f32_16x16x4_f32 (fp32 operands)"}
     return out
 
 

@@ -288,10 +288,13 @@ int hiprwkv_wkv6_fwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64
   A.io_f32 = io_dtype == HIPRWKV_F32; A.st_f32 = state_dtype == HIPRWKV_F32;
   A.flags = flags;
   A.status = status_word();
-  const bool chunked = io_dtype == HIPRWKV_BF16 && !(flags & HIPRWKV_FORCE_SEQ);
+  // chunked matrix-core kernels (fp16 operands for bf16 I/O, fp32 operands for fp32 I/O) unless HIPRWKV_FORCE_SEQ
+  const bool chunked = !(flags & HIPRWKV_FORCE_SEQ);
   const bool small_t = T <= HIPRWKV_SMALL_T && !(flags & HIPRWKV_NO_SMALL_T);
   hipStream_t st = static_cast<hipStream_t>(stream);
-  hipError_t e = small_t ? launch_wkv6_small_t_fwd(A, st) : chunked ? launch_wkv6_chunk_fwd(A, st) : launch_wkv6_seq_fwd(A, st);
+  hipError_t e = small_t ? launch_wkv6_small_t_fwd(A, st)
+               : !chunked ? launch_wkv6_seq_fwd(A, st)
+               : A.io_f32 ? launch_wkv6_chunk_fwd_f32(A, st) : launch_wkv6_chunk_fwd(A, st);
   if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "wkv6_fwd: %s", hipGetErrorString(e));
   return HIPRWKV_OK;
 }

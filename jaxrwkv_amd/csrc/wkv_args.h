@@ -106,6 +106,7 @@ hipError_t launch_wkv7_seq_bwd_b(const Wkv7Args& A, hipStream_t stream);
 hipError_t launch_wkv7_seq_bwd_c(const Wkv7Args& A, hipStream_t stream);
 hipError_t launch_wkv6_seq_fwd(const Wkv6Args& A, hipStream_t stream);
 hipError_t launch_wkv6_chunk_fwd(const Wkv6Args& A, hipStream_t stream);
+hipError_t launch_wkv6_chunk_fwd_f32(const Wkv6Args& A, hipStream_t stream);
 hipError_t launch_wkv6_seq_bwd(const Wkv6Args& A, hipStream_t stream);
 hipError_t launch_wkv6_chunk_bwd_f(const Wkv6Args& A, hipStream_t stream);
 hipError_t launch_wkv6_chunk_bwd_r(const Wkv6Args& A, hipStream_t stream);

@@ -99,6 +99,22 @@ def test_wkv6(case):
         assert_close("new_s", new_s, ref_s)
 
 
+@pytest.mark.parametrize("case", CASES, ids=lambda c: "B{B}-T{T}-H{H}-p{p}-c{compat:d}-f{frac}".format(**c))
+def test_wkv6_fp32(case):
+    """fp32 I/O: the chunked forward kernel on fp32 matrix instructions and the sequential one at the fp32 bar."""
+    from tests import test_gpu_wkv6 as t6
+    B, T, H, compat = case["B"], case["T"], case["H"], case["compat"]
+    x = wkv6_inputs(B, T, H, 64, seed=case["seed"], p_reset=case["p"])
+    if case["frac"] == 0.0:
+        x["length"][0] = 0
+    ref_s, ref_y = o6.wkv6_base(x["r"], x["k"], x["v"], x["w"], x["u"], x["s"], x["length"], x["new_starts"],
+                                compat=compat)
+    for force_seq in (False, True):
+        new_s, y = t6.run_fwd(x, torch.float32, compat, force_seq)
+        assert_close("y", y, ref_y)
+        assert_close("new_s", new_s, ref_s)
+
+
 @pytest.mark.parametrize("case", CASES, ids=lambda c: "B{B}-T{T}-C{C}-p{p}-c{compat:d}-f{frac}".format(**c))
 def test_wkv4(case):
     B, T, C, compat = case["B"], case["T"], case["C"], case["compat"]

@@ -13,11 +13,11 @@ pytestmark = pytest.mark.gpu
 GOLD = os.path.join(os.path.dirname(__file__), "golden", "wkv6_small.npz")
 
 
-def run_fwd(x, dtype, compat):
+def run_fwd(x, dtype, compat, force_seq=False):
     from jaxrwkv_amd import ops
     new_s, y = ops.wkv6_fwd(dev(x["r"], dtype), dev(x["k"], dtype), dev(x["v"], dtype), dev(x["w"], dtype),
                             dev(x["u"], dtype), dev(x["s"]), dev(x["length"]), dev(x["new_starts"]), compat=compat,
-                            small_t=False)
+                            small_t=False, force_seq=force_seq)
     torch.cuda.synchronize()
     return host(new_s), host(y)
 
@@ -43,16 +43,18 @@ def test_fp32_golden_fixture(compat):
         assert_close("g" + n, g, z[f"g{n}_c{c}"], scale_atol=True)
 
 
-@pytest.mark.parametrize("B,T,H,seed", [(1, 1, 1, 0), (2, 17, 3, 1), (1, 33, 2, 3), (3, 100, 2, 4), (2, 257, 4, 5)])
+# fp32 I/O runs on the chunked kernel with fp32 matrix operands by default and on the sequential kernel with force_seq
+@pytest.mark.parametrize("force_seq", [False, True], ids=["chunked", "seq"])
+@pytest.mark.parametrize("B,T,H,seed", [(1, 1, 1, 0), (2, 17, 3, 1), (1, 33, 2, 3), (3, 100, 2, 4), (2, 257, 4, 5), (1, 1000, 1, 6)])
 @pytest.mark.parametrize("compat", [True, False])
-def test_fp32_forward_shapes(B, T, H, seed, compat):
+def test_fp32_forward_shapes(B, T, H, seed, compat, force_seq):
     x = wkv6_inputs(B, T, H, 64, seed=seed, p_reset=0.05)
     if T > 4:
         x["new_starts"][0, 0] = True
         x["length"][0] = T // 2
         x["new_starts"][0, T // 2] = True
     ref_s, ref_y = o6.wkv6_base(x["r"], x["k"], x["v"], x["w"], x["u"], x["s"], x["length"], x["new_starts"], compat=compat)
-    new_s, y = run_fwd(x, torch.float32, compat)
+    new_s, y = run_fwd(x, torch.float32, compat, force_seq)
     assert_close("y", y, ref_y)
     assert_close("new_s", new_s, ref_s)
 
