@@ -410,6 +410,17 @@ def bench_wkv6(torch, ops, args):
         out["fp32_io"] = {"kernel_ms": kc, "tokens_per_s": tokens / (kc * 1e-3),
                           "hbm_frac": b32 / (kc * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": b32,
                           "sequential_kernel_ms": ks, "kernel": "chunked, v_mfma_f32_16x16x4_f32 (fp32 operands)"}
+        if not args.no_bwd:
+            dy32 = dy.float()
+
+            def fb32(fs):
+                ops.wkv6_fwd(r32, k32, v32, w32, u32, s, None, ns, compat=True, force_seq=fs)
+                return ops.wkv6_bwd(r32, k32, v32, w32, u32, s, None, ns, dy32, None, compat=True, force_seq=fs)
+            n4 = max(2, args.steps // 10)
+            wc, _ = time_region(torch, lambda: fb32(False), n4, 1)
+            wsq, _ = time_region(torch, lambda: fb32(True), n4, 1)
+            out["fp32_io"]["fwd_bwd_ms"] = 1e3 * wc / n4
+            out["fp32_io"]["sequential_fwd_bwd_ms"] = 1e3 * wsq / n4
     return out
 
 

@@ -177,7 +177,8 @@ size_t hiprwkv_wkv6_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t
 
 /* Cotangents of wkv6_fwd: gr,gk,gv,gw (B,T,H,N) io_dtype; gu (B,H,N) fp32, to be summed
  * over B by the caller (as the reference does for the WKV4 parameters, rwkv4.py:351);
- * gs (B,H,N,N) state_dtype. */
+ * gs (B,H,N,N) state_dtype.  Forward and backward run on the matrix cores for both I/O
+ * dtypes (fp32 operands beside fp32 I/O); HIPRWKV_FORCE_SEQ selects the sequential kernels. */
 int hiprwkv_wkv6_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype,
                      int64_t B, int64_t T, int64_t H, int64_t N,
                      const void* r, const void* k, const void* v, const void* w,

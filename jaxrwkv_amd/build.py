@@ -9,7 +9,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libhiprwkv.so")
-SOURCES = ["api.hip", "wkv7_seq.hip", "wkv7_fwd.hip", "wkv7_fwd_f32.hip", "wkv7_bwd_a.hip", "wkv7_chunk_bwd_b.hip", "wkv7_chunk_bwd_c.hip", "wkv7_bwd_a_f32.hip", "wkv7_bwd_b_f32.hip", "wkv7_bwd_c_f32.hip", "wkv7_small_t.hip", "wkv6_seq.hip", "wkv6_small_t.hip", "wkv6_fwd.hip", "wkv6_fwd_f32.hip", "wkv6_chunk_bwd_f.hip", "wkv6_chunk_bwd_r.hip", "wkv4.hip", "rwkv7_mix.hip", "rwkv7_shift.hip", "rwkv7_gates.hip"]
+SOURCES = ["api.hip", "wkv7_seq.hip", "wkv7_fwd.hip", "wkv7_fwd_f32.hip", "wkv7_bwd_a.hip", "wkv7_chunk_bwd_b.hip", "wkv7_chunk_bwd_c.hip", "wkv7_bwd_a_f32.hip", "wkv7_bwd_b_f32.hip", "wkv7_bwd_c_f32.hip", "wkv7_small_t.hip", "wkv6_seq.hip", "wkv6_small_t.hip", "wkv6_fwd.hip", "wkv6_fwd_f32.hip", "wkv6_chunk_bwd_f.hip", "wkv6_chunk_bwd_r.hip", "wkv6_bwd_f_f32.hip", "wkv6_bwd_r_f32.hip", "wkv4.hip", "rwkv7_mix.hip", "rwkv7_shift.hip", "rwkv7_gates.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared", "-fno-gpu-rdc",
     # packed-fp32 VALU forms are switched off on purpose for this GPU pool

@@ -365,15 +365,18 @@ int hiprwkv_wkv6_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype, int64
   char* ws = static_cast<char*>(workspace);
   A.er = reinterpret_cast<float*>(at_phase(ws, r, 5));
   A.eI = reinterpret_cast<float*>(reinterpret_cast<char*>(A.er) + align256((size_t)B * T * H * N * sizeof(float)));
-  // Two sweeps: F (forward) -> gr, gu, er, eI; R (reverse) -> gk, gv, gw, gs.  bf16 I/O runs them on the chunked
-  // MFMA kernels.
+  // Two sweeps: F (forward) -> gr, gu, er, eI; R (reverse) -> gk, gv, gw, gs, on the chunked matrix-core kernels
+  // (bf16 pairs for bf16 I/O, fp32 operands for fp32 I/O); HIPRWKV_FORCE_SEQ selects the sequential kernel.
   hipStream_t st = static_cast<hipStream_t>(stream);
   hipError_t e;
-  if (io_dtype == HIPRWKV_BF16 && !(flags & HIPRWKV_FORCE_SEQ)) {
+  if (flags & HIPRWKV_FORCE_SEQ) {
+    e = launch_wkv6_seq_bwd(A, st);
+  } else if (A.io_f32) {
+    e = launch_wkv6_chunk_bwd_f_f32(A, st);
+    if (e == hipSuccess) e = launch_wkv6_chunk_bwd_r_f32(A, st);
+  } else {
     e = launch_wkv6_chunk_bwd_f(A, st);
     if (e == hipSuccess) e = launch_wkv6_chunk_bwd_r(A, st);
-  } else {
-    e = launch_wkv6_seq_bwd(A, st);
   }
   if (e != hipSuccess) return fail(HIPRWKV_ELAUNCH, "wkv6_bwd: %s", hipGetErrorString(e));
   return HIPRWKV_OK;

@@ -110,6 +110,8 @@ hipError_t launch_wkv6_chunk_fwd_f32(const Wkv6Args& A, hipStream_t stream);
 hipError_t launch_wkv6_seq_bwd(const Wkv6Args& A, hipStream_t stream);
 hipError_t launch_wkv6_chunk_bwd_f(const Wkv6Args& A, hipStream_t stream);
 hipError_t launch_wkv6_chunk_bwd_r(const Wkv6Args& A, hipStream_t stream);
+hipError_t launch_wkv6_chunk_bwd_f_f32(const Wkv6Args& A, hipStream_t stream);
+hipError_t launch_wkv6_chunk_bwd_r_f32(const Wkv6Args& A, hipStream_t stream);
 hipError_t launch_wkv4_fwd(const Wkv4Args& A, hipStream_t stream);
 hipError_t launch_wkv4_bwd(const Wkv4Args& A, hipStream_t stream);
 hipError_t launch_rwkv7_premix(int io_f32, int64_t rows, int64_t H, const void* k, const void* a, const void* k_k,

@@ -293,9 +293,10 @@ def wkv6_bwd(r, k, v, w, u, s, length, new_starts, gy, gs_out=None, compat=True,
 
 class _Wkv6(torch.autograd.Function):
     @staticmethod
-    def forward(ctx, r, k, v, w, u, s, length, new_starts, compat):
-        new_s, y = wkv6_fwd(r, k, v, w, u, s, length, new_starts, compat)
+    def forward(ctx, r, k, v, w, u, s, length, new_starts, compat, force_seq):
+        new_s, y = wkv6_fwd(r, k, v, w, u, s, length, new_starts, compat, force_seq=force_seq)
         ctx.compat = compat
+        ctx.force_seq = force_seq
         ctx.shapes = (w.shape, u.shape)
         ctx.save_for_backward(r, k, v, w, u, s, length, new_starts)
         return new_s, y
@@ -305,15 +306,15 @@ class _Wkv6(torch.autograd.Function):
         r, k, v, w, u, s, length, new_starts = ctx.saved_tensors
         if gy is None:
             gy = torch.zeros_like(r)
-        gr, gk, gv, gw, gu, gs = wkv6_bwd(r, k, v, w, u, s, length, new_starts, gy, gs_out, ctx.compat)
-        return gr, gk, gv, gw.reshape(ctx.shapes[0]), gu.reshape(ctx.shapes[1]), gs, None, None, None
+        gr, gk, gv, gw, gu, gs = wkv6_bwd(r, k, v, w, u, s, length, new_starts, gy, gs_out, ctx.compat, ctx.force_seq)
+        return gr, gk, gv, gw.reshape(ctx.shapes[0]), gu.reshape(ctx.shapes[1]), gs, None, None, None, None
 
 
-def wkv6(r, k, v, w, u, s, length=None, new_starts=None, compat=True):
-    """Differentiable WKV6: returns (new_s, y)."""
+def wkv6(r, k, v, w, u, s, length=None, new_starts=None, compat=True, force_seq=False):
+    """Differentiable WKV6: returns (new_s, y).  ``force_seq`` runs the sequential fp32 kernels whatever the dtype."""
     B, T = r.shape[:2]
     length, new_starts = _length_ns(length, new_starts, B, T, r.device)
-    return _Wkv6.apply(r, k, v, w, u, s, length, new_starts, compat)
+    return _Wkv6.apply(r, k, v, w, u, s, length, new_starts, compat, force_seq)
 
 
 # ----------------------------------------------------------------------------- WKV4

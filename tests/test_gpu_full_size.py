@@ -117,6 +117,31 @@ def test_wkv6_chunked_equals_sequential_at_the_benchmark_shape():
         assert rel_rms(c, q) < tol[n_], (n_, rel_rms(c, q))
 
 
+def test_wkv6_fp32_chunked_equals_sequential_at_the_benchmark_shape():
+    """fp32 I/O at B=16 T=2048 H=32: the chunked kernels on fp32 matrix instructions against the sequential fp32
+    kernels, forward and all six cotangents; both compute in fp32 throughout."""
+    from jaxrwkv_amd import ops
+    B, T, H, N = 16, 2048, 32, 64
+    g = torch.Generator("cuda").manual_seed(7)
+    n = lambda *s: torch.randn(s, device="cuda", generator=g)
+    r, k, v, dy = (n(B, T, H, N) for _ in range(4))
+    w = -torch.exp(-0.5 + 0.5 * n(B, T, H, N))
+    u = 0.5 * n(H, N)
+    s = 0.1 * n(B, H, N, N)
+    ns = torch.rand((B, T), device="cuda", generator=g) < 1.0 / 512
+    length = torch.randint(T // 2, T + 1, (B,), device="cuda", generator=g, dtype=torch.int32)
+    ds = n(B, H, N, N)
+    out = {}
+    for fs in (False, True):
+        new_s, y = ops.wkv6_fwd(r, k, v, w, u, s, length, ns, compat=True, force_seq=fs)
+        out[fs] = (new_s, y) + tuple(ops.wkv6_bwd(r, k, v, w, u, s, length, ns, dy, ds, compat=True, force_seq=fs))
+    torch.cuda.synchronize()
+    names = ("new_s", "y", "gr", "gk", "gv", "gw", "gu", "gs")
+    for n_, c, q in zip(names, out[False], out[True]):
+        assert c.dtype == torch.float32 and torch.isfinite(c).all(), n_
+        assert rel_rms(c, q) < (1e-4 if n_ == "gw" else 1e-5), (n_, rel_rms(c, q))
+
+
 def test_wkv4_split_call_equals_single_call_at_the_benchmark_shape():
     from jaxrwkv_amd import ops
     B, T, C = 32, 4096, 2560

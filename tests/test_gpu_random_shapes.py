@@ -101,7 +101,8 @@ def test_wkv6(case):
 
 @pytest.mark.parametrize("case", CASES, ids=lambda c: "B{B}-T{T}-H{H}-p{p}-c{compat:d}-f{frac}".format(**c))
 def test_wkv6_fp32(case):
-    """fp32 I/O: the chunked forward kernel on fp32 matrix instructions and the sequential one at the fp32 bar."""
+    """fp32 I/O: the chunked kernels on fp32 matrix instructions and the sequential ones, forward and backward, at the
+    fp32 bar."""
     from tests import test_gpu_wkv6 as t6
     B, T, H, compat = case["B"], case["T"], case["H"], case["compat"]
     x = wkv6_inputs(B, T, H, 64, seed=case["seed"], p_reset=case["p"])
@@ -113,6 +114,11 @@ def test_wkv6_fp32(case):
         new_s, y = t6.run_fwd(x, torch.float32, compat, force_seq)
         assert_close("y", y, ref_y)
         assert_close("new_s", new_s, ref_s)
+    ref = o6.wkv6_bwd(x["r"], x["k"], x["v"], x["w"], x["u"], x["s"], x["length"], x["new_starts"], x["dy"], x["ds"],
+                      compat=compat)
+    for force_seq in (False, True):      # the two sweeps on fp32 matrix instructions, and the sequential kernel
+        for n, g, rf in zip("rkvwus", t6.run_bwd(x, torch.float32, compat, force_seq), ref):
+            assert_close("g" + n, g, rf, atol=t6.GRAD_ATOL[n], scale_atol=True)
 
 
 @pytest.mark.parametrize("case", CASES, ids=lambda c: "B{B}-T{T}-C{C}-p{p}-c{compat:d}-f{frac}".format(**c))

@@ -11,6 +11,10 @@ from tests.inputs import wkv6_inputs
 
 pytestmark = pytest.mark.gpu
 GOLD = os.path.join(os.path.dirname(__file__), "golden", "wkv6_small.npz")
+# Cotangents: rtol 1e-4 and atol 1e-5 x max(1, rms of the reference tensor).  The decay gradient is a running sum over
+# the rest of the sequence of terms that cancel (er_t - k_t.(G_t v_t)), each an fp32 result: 5e-5 of its rms (measured
+# up to 1.1e-5 for the chunked sweeps on fp32 matrix instructions, whose G v passes through 1/E_t, at 255 tokens).
+GRAD_ATOL = dict(r=1e-5, k=1e-5, v=1e-5, w=5e-5, u=1e-5, s=1e-5)
 
 
 def run_fwd(x, dtype, compat, force_seq=False):
@@ -22,11 +26,12 @@ def run_fwd(x, dtype, compat, force_seq=False):
     return host(new_s), host(y)
 
 
-def run_bwd(x, dtype, compat):
+def run_bwd(x, dtype, compat, force_seq=False):
     from jaxrwkv_amd import ops
     t = {n: dev(x[n], dtype).requires_grad_() for n in ("r", "k", "v", "w", "u")}
     s = dev(x["s"]).requires_grad_()
-    new_s, y = ops.wkv6(t["r"], t["k"], t["v"], t["w"], t["u"], s, dev(x["length"]), dev(x["new_starts"]), compat=compat)
+    new_s, y = ops.wkv6(t["r"], t["k"], t["v"], t["w"], t["u"], s, dev(x["length"]), dev(x["new_starts"]), compat=compat,
+                        force_seq=force_seq)
     ((y.float() * dev(x["dy"])).sum() + (new_s * dev(x["ds"])).sum()).backward()
     torch.cuda.synchronize()
     return [host(t[n].grad) for n in ("r", "k", "v", "w", "u")] + [host(s.grad)]
@@ -59,15 +64,16 @@ def test_fp32_forward_shapes(B, T, H, seed, compat, force_seq):
     assert_close("new_s", new_s, ref_s)
 
 
+@pytest.mark.parametrize("force_seq", [False, True], ids=["chunked", "seq"])
 @pytest.mark.parametrize("compat", [True, False])
-@pytest.mark.parametrize("B,T,H,seed", [(2, 48, 2, 21), (1, 97, 3, 22)])
-def test_fp32_backward(B, T, H, seed, compat):
+@pytest.mark.parametrize("B,T,H,seed", [(2, 48, 2, 21), (1, 97, 3, 22), (1, 500, 2, 24)])
+def test_fp32_backward(B, T, H, seed, compat, force_seq):
     x = wkv6_inputs(B, T, H, 64, seed=seed, p_reset=0.04)
     x["length"][0] = T // 2
     x["new_starts"][0, T // 2] = True
     ref = o6.wkv6_bwd(x["r"], x["k"], x["v"], x["w"], x["u"], x["s"], x["length"], x["new_starts"], x["dy"], x["ds"], compat=compat)
-    for n, g, rf in zip("rkvwus", run_bwd(x, torch.float32, compat), ref):
-        assert_close("g" + n, g, rf, scale_atol=True)
+    for n, g, rf in zip("rkvwus", run_bwd(x, torch.float32, compat, force_seq), ref):
+        assert_close("g" + n, g, rf, atol=GRAD_ATOL[n], scale_atol=True)
 
 
 def test_length_zero():
