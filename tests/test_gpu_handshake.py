@@ -89,3 +89,50 @@ def test_wkv7_fp32_forward_poisons_its_outputs_and_counts():
     assert ops.handshake_failures() == before
     for a_, b_ in zip(again, good):
         assert torch.equal(a_, b_)
+
+
+def test_wkv7_fp32_backward_poisons_its_outputs_and_counts():
+    from jaxrwkv_amd import _lib, ops
+    args, dy, ds = inputs7(seed=3)
+    args = tuple(t.float() if isinstance(t, torch.Tensor) else t for t in args)
+    dy = dy.float()
+    good = ops.wkv7_fwd(*args, want_sa=True)
+    ref = ops.wkv7_bwd(*args, dy, good[2], ds)
+    before = ops.handshake_failures()
+    grads = ops.wkv7_bwd(*args, dy, good[2], ds, debug_flags=_lib.DEBUG_DROP_PUBLISH)
+    assert ops.handshake_failures() - before == 3 * B * H          # three sweeps
+    for g in grads:
+        assert g.dtype == torch.float32 and all_nan(g)
+    before = ops.handshake_failures()
+    again = ops.wkv7_bwd(*args, dy, good[2], ds)
+    assert ops.handshake_failures() == before
+    for a_, b_ in zip(again, ref):
+        assert torch.equal(a_, b_)
+
+
+def test_wkv6_fp32_forward_and_backward_poison_their_outputs_and_count():
+    from jaxrwkv_amd import _lib, ops
+    g = torch.Generator("cuda").manual_seed(4)
+    n = lambda *s: torch.randn(s, device="cuda", generator=g)
+    r, k, v, dy = (n(B, T, H, N) for _ in range(4))
+    w = -torch.exp(-0.5 + 0.5 * n(B, T, H, N))
+    u = 0.5 * n(H, N)
+    s, ds = 0.1 * n(B, H, N, N), n(B, H, N, N)
+    good = ops.wkv6_fwd(r, k, v, w, u, s)
+    ref = ops.wkv6_bwd(r, k, v, w, u, s, None, None, dy, ds)
+    before = ops.handshake_failures()
+    new_s, y = ops.wkv6_fwd(r, k, v, w, u, s, debug_flags=_lib.DEBUG_DROP_PUBLISH)
+    assert ops.handshake_failures() - before == B * H
+    assert y.dtype == torch.float32 and all_nan(new_s) and all_nan(y)
+    before = ops.handshake_failures()
+    grads = ops.wkv6_bwd(r, k, v, w, u, s, None, None, dy, ds, debug_flags=_lib.DEBUG_DROP_PUBLISH)
+    assert ops.handshake_failures() - before == 2 * B * H          # two sweeps
+    for t in grads:
+        assert all_nan(t)
+    before = ops.handshake_failures()
+    again = ops.wkv6_fwd(r, k, v, w, u, s)
+    g2 = ops.wkv6_bwd(r, k, v, w, u, s, None, None, dy, ds)
+    assert ops.handshake_failures() == before
+    assert torch.equal(again[0], good[0]) and torch.equal(again[1], good[1])
+    for a_, b_ in zip(g2, ref):
+        assert torch.equal(a_, b_)
