@@ -158,6 +158,8 @@ __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags
   float bonus = 0.f;
 #pragma unroll
   for (int hf = 0; hf < 2; ++hf) {
+    // issue priority rises with the wave's progress through the chunk (see wkv7_fwd.hip)
+    if (hf == 0) __builtin_amdgcn_s_setprio(1); else __builtin_amdgcn_s_setprio(2);
     {
       float fv[8];
       unpack8(x.v[hf], fv);
@@ -258,6 +260,7 @@ __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags
     M = mfma(kh_h, qt_l, M);
     M = mfma(kh_l, qt_h, M);
   }
+  __builtin_amdgcn_s_setprio(3);
   // ---- bonus of token t summed over the four key groups
   bonus += __shfl_xor(bonus, 16, 64);
   bonus += __shfl_xor(bonus, 32, 64);
@@ -292,6 +295,7 @@ __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags
     slot->keep_end = (lastseg == 0) ? 1 : 0;
     slot->keep_snap = (F.snap >= 0 && (!slow || seg_of(resets, F.snap) == 0)) ? 1 : 0;
   }
+  __builtin_amdgcn_s_setprio(0);
 }
 
 // ---------------------------------------------------------------------------------------------------- consumer

@@ -155,6 +155,8 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
   f32x4_t G1 = zero4, G2 = zero4, G3 = zero4;   // qt_m.bh_n, at_m.kh_n, qt_m.kh_n
 #pragma unroll
   for (int hf = 0; hf < 2; ++hf) {
+    // issue priority rises with the wave's progress through the chunk (see wkv7_fwd.hip)
+    if (hf == 0) __builtin_amdgcn_s_setprio(1); else __builtin_amdgcn_s_setprio(2);
     // ---- v^T (dy^T) of value tiles 2hf, 2hf+1: D[token][value] = sum_k V[token][k] sel[k][value]
     {
       uint4 vr = x.v[hf];
@@ -288,6 +290,7 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
       G3 = mfma(qA, kB, G3);      // Mkr^T[m][n] = qt_m . kh_n
     }
   }
+  __builtin_amdgcn_s_setprio(3);
   // ---- triangular masks: later rows m for column n
   const int n = t;
   auto mask_tiles = [&](int i, bool lt, bool le, bool gt, bool ge) {
@@ -341,6 +344,7 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
     slot->keep_end = (lastseg == 0) ? 1 : 0;
     slot->keep_snap = (F.snap >= 0 && (!slow || seg_of(F.ns, F.snap) == 0)) ? 1 : 0;
   }
+  __builtin_amdgcn_s_setprio(0);
 }
 
 // ---------------------------------------------------------------------------------------------------- consumer

@@ -138,8 +138,14 @@ __device__ __forceinline__ uint4 pack_h8(const float (&f)[8]) {
 
 // Everything of one chunk that does not depend on the carried state.  The two 32-key halves go through the same
 // pipeline one after the other, which keeps the live register set small.
+//
+// With `staged` the wave raises its issue priority as it advances through the chunk (1, 2, then 3 for the inverse; 0
+// again while it requests the next operands and waits for a slot).  At equal priority the SIMD serves its oldest wave
+// first: time stamps showed the youngest of the three producers of a SIMD taking 10 000 cycles for a chunk and the
+// oldest 6 000, and the chunks are consumed in order, so the slow one set the pace.  Measured: 4 % faster without
+// the `sa` output, 1.5-2 % slower with it (whatever the steps), so the launch that writes `sa` goes without.
 __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags& F, Slot* __restrict__ slot,
-                                        SnapSlot* __restrict__ snap, unsigned* events) {
+                                        SnapSlot* __restrict__ snap, unsigned* events, bool staged) {
   const int t = lane & 15, g = lane >> 4;
   const bool valid = t < F.nvalid;
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -174,6 +180,9 @@ __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags
   f32x4_t G1 = zero4, G2 = zero4, G3 = zero4;   // Mka, Mbr, Mkr
 #pragma unroll
   for (int hf = 0; hf < 2; ++hf) {
+    if (staged) {
+      if (hf == 0) __builtin_amdgcn_s_setprio(1); else __builtin_amdgcn_s_setprio(2);
+    }
     // ---- v in fp16, row-major (the consumers read it transposed)
     {
       float fv[8];
@@ -307,6 +316,7 @@ __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags
       G3 = mfma(kA, qB, G3);        // Mkr[m][n] = kh_m . qt_n
     }
   }
+  if (staged) __builtin_amdgcn_s_setprio(3);
   // ---- triangular masks: earlier rows m for column n
   const int n = t;
   auto mask_tiles = [&](int i, bool lt, bool le, bool gt) {
@@ -362,6 +372,7 @@ __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags
     slot->keep_end = (lastseg == 0) ? 1 : 0;
     slot->keep_snap = (F.snap >= 0 && (!slow || seg_of(F.ns, F.snap) == 0)) ? 1 : 0;
   }
+  if (staged) __builtin_amdgcn_s_setprio(0);
 }
 
 // ---------------------------------------------------------------------------------------------------- consumer
@@ -634,7 +645,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_fwd_kernel(Wkv7Args
       Slot* slot = &slots[si];
       if (j >= RING && !wait_consumed_lazy(sy, si, j - RING + 1, lane)) break;
       mask_raw(raw, F.nvalid, lane);
-      produce(lane, raw, F, slot, snapslot, events_word(A.status));
+      produce(lane, raw, F, slot, snapslot, events_word(A.status), A.sa == nullptr);
       if (j + NPROD < nch) {
         load_raw(raw, A, b, h, c0 + (int64_t)NPROD * CK, lane);
         ns_mine = chunk_flag_prefetch(A.ns, A.T, b, c0 + (int64_t)NPROD * CK, lane);
