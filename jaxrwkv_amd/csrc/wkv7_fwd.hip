@@ -378,9 +378,27 @@ __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags
 // ---------------------------------------------------------------------------------------------------- consumer
 // Wave q holds S^T for value rows 16q..16q+15 as four 16x16 accumulator tiles: lane (n = lane%16, g = lane/16),
 // S[tile][i] = S[value 16q+n][key 16*tile + 4g + i].
+// Byte offsets of this lane's operands inside a slot, computed once (the asm statement keeps the compiler from
+// recomputing them from the lane index in every chunk).
+struct LaneOffs {
+  uint32_t aq, l8, l16, vv, upd, gm;
+};
+__device__ __forceinline__ LaneOffs lane_offs(int q, int lane) {
+  const int n = lane & 15, g = lane >> 4;
+  LaneOffs o;
+  o.aq = (uint32_t)(offsetof(Slot, AQ) + (n * RS + 8 * g) * 2);
+  o.l8 = (uint32_t)(offsetof(Slot, P) + lane * 8);
+  o.l16 = (uint32_t)(offsetof(Slot, BrKr) + lane * 16);
+  o.vv = (uint32_t)(offsetof(Slot, V) + ((4 * g + (n >> 2)) * RS + 16 * q + 4 * (n & 3)) * 2);
+  o.upd = (uint32_t)(offsetof(Slot, BK) + ((4 * g + (n >> 2)) * RS + 4 * (n & 3)) * 2);
+  o.gm = (uint32_t)(offsetof(Slot, gamma) + 16 * g);
+  asm volatile("" : "+v"(o.aq), "+v"(o.l8), "+v"(o.l16), "+v"(o.vv), "+v"(o.upd), "+v"(o.gm));
+  return o;
+}
 struct Consumer {
   f32x4_t S[4];
   int q, lane;
+  LaneOffs off;
 };
 
 // Operands a consumer fetches a chunk ahead: everything the W / SA / Y chain reads.
@@ -393,18 +411,18 @@ struct Ops {
   int keep_end;
 };
 
-__device__ __forceinline__ void load_ops(Ops& o, const Slot* __restrict__ slot, int q, int lane) {
-  const int n = lane & 15, g = lane >> 4;
+__device__ __forceinline__ void load_ops(Ops& o, const Slot* __restrict__ slot, const LaneOffs& f) {
+  const char* const sb = reinterpret_cast<const char*>(slot);
 #pragma unroll
   for (int ar = 0; ar < 2; ++ar)
 #pragma unroll
     for (int j = 0; j < 2; ++j)
-      o.aq[ar][j] = *reinterpret_cast<const u32x4_t*>(&slot->AQ[ar][n][32 * j + 8 * g]);
-  o.P = slot->P[lane];
-  o.Ka = slot->Ka[lane];
-  o.BrKr = slot->BrKr[lane];
-  o.KrLo = slot->KrLo[lane];
-  o.vv = lds_tr4(&slot->V[4 * g + (n >> 2)][16 * q + 4 * (n & 3)]);
+      o.aq[ar][j] = *reinterpret_cast<const u32x4_t*>(sb + f.aq + ar * (CK * RS * 2) + j * 64);
+  o.P = *reinterpret_cast<const u32x2_t*>(sb + f.l8);
+  o.Ka = *reinterpret_cast<const u32x2_t*>(sb + f.l8 + (offsetof(Slot, Ka) - offsetof(Slot, P)));
+  o.BrKr = *reinterpret_cast<const u32x4_t*>(sb + f.l16);
+  o.KrLo = *reinterpret_cast<const u32x2_t*>(sb + f.l8 + (offsetof(Slot, KrLo) - offsetof(Slot, P)));
+  o.vv = lds_tr4(reinterpret_cast<const uint16_t*>(sb + f.vv));
   o.keep_end = slot->keep_end;
 }
 
@@ -461,8 +479,11 @@ __device__ __forceinline__ bool consume(Consumer& C, Ops& o, const Slot* __restr
   float4 gm[4];
 #pragma unroll
   for (int tile = 0; tile < 4; ++tile) {
-    up[tile] = load_upd(slot->BK, tile, lane);
-    gm[tile] = *reinterpret_cast<const float4*>(&slot->gamma[16 * tile + 4 * g]);
+    const char* const sb = reinterpret_cast<const char*>(slot);
+    const u32x2_t be = lds_tr4(reinterpret_cast<const uint16_t*>(sb + C.off.upd + 32 * tile));
+    const u32x2_t ke = lds_tr4(reinterpret_cast<const uint16_t*>(sb + C.off.upd + CK * RS * 2 + 32 * tile));
+    up[tile] = u32x4_t{be[0], be[1], ke[0], ke[1]};
+    gm[tile] = *reinterpret_cast<const float4*>(sb + C.off.gm + 64 * tile);
   }
   const bool keep_end = __builtin_amdgcn_readfirstlane(o.keep_end) != 0;
   // B operands from the state: MFMA j contracts over the keys of tiles 2j and 2j+1
@@ -489,7 +510,7 @@ __device__ __forceinline__ bool consume(Consumer& C, Ops& o, const Slot* __restr
   bool ok = true;
   if (next != nullptr) {
     ok = next_ready(peeked);
-    load_ops(o, next, C.q, lane);
+    load_ops(o, next, C.off);
   }
   // state snapshot for `length` (one chunk per sequence)
   if (is_snap) {
@@ -592,6 +613,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_fwd_kernel(Wkv7Args
     Consumer C;
     C.q = cq;
     C.lane = lane;
+    C.off = lane_offs(cq, lane);
     const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int tile = 0; tile < 4; ++tile) C.S[tile] = load_state_tile(A.s, A.st_f32, state_off(A, b, h, cq, lane, tile));
@@ -612,11 +634,12 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_fwd_kernel(Wkv7Args
     bool ok = true;
     if (nch > 0) {
       ok = wait_ready(sy, 0, 1);
-      load_ops(ops, &slots[0], cq, lane);
+      load_ops(ops, &slots[0], C.off);
     }
+    int si = 0;                       // j % RING, kept by counting
     for (int j = 0; j < nch && ok; ++j) {
       const int nvalid = (j + 1 < nch || A.T % CK == 0) ? CK : (int)(A.T % CK);
-      const int si = j % RING, sn = (j + 1) % RING;
+      const int sn = (si + 1 == RING) ? 0 : si + 1;
       const Slot* next = (j + 1 < nch) ? &slots[sn] : nullptr;
       ok = consume(C, ops, &slots[si], next, snapslot, A, b, h, nvalid, j == csnap, q2drop, oc,
                    [&]() { return peek_ready(sy, sn); },
@@ -625,6 +648,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_fwd_kernel(Wkv7Args
                    });
       // every LDS read of slot si has returned: its data went into the MFMAs above
       if (lane == 0) __hip_atomic_store(&sy->consumed[cq][si], j + 1, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP);
+      si = sn;
     }
     // an operand beyond the fp16 range leaves inf or NaN in the carried state (until a reset discards it): count it
     count_nonfinite(C.S, lane, events_word(A.status));
