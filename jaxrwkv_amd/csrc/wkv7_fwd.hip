@@ -139,13 +139,13 @@ __device__ __forceinline__ uint4 pack_h8(const float (&f)[8]) {
 // Everything of one chunk that does not depend on the carried state.  The two 32-key halves go through the same
 // pipeline one after the other, which keeps the live register set small.
 //
-// With `staged` the wave raises its issue priority as it advances through the chunk (1, 2, then 3 for the inverse; 0
-// again while it requests the next operands and waits for a slot).  At equal priority the SIMD serves its oldest wave
-// first: time stamps showed the youngest of the three producers of a SIMD taking 10 000 cycles for a chunk and the
-// oldest 6 000, and the chunks are consumed in order, so the slow one set the pace.  Measured: 4 % faster without
-// the `sa` output, 1.5-2 % slower with it (whatever the steps), so the launch that writes `sa` goes without.
+// Issue priorities: at equal priority a SIMD serves its oldest wave first, and time stamps show the youngest of the
+// three producers of a SIMD taking 10 000 cycles for a chunk where the oldest takes 6 000.  Raising a producer's
+// priority as it advances through its chunk evens that out and makes an isolated launch 4 % faster, but launches
+// issued back to back (the GPU at its power limit) 2.8 % slower, so this kernel's producers stay at the default
+// priority; the WKV6 forward, where the same steps gain 3.5 % back to back, has them.
 __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags& F, Slot* __restrict__ slot,
-                                        SnapSlot* __restrict__ snap, unsigned* events, bool staged) {
+                                        SnapSlot* __restrict__ snap, unsigned* events) {
   const int t = lane & 15, g = lane >> 4;
   const bool valid = t < F.nvalid;
   const f32x4_t zero4 = {0.f, 0.f, 0.f, 0.f};
@@ -180,9 +180,6 @@ __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags
   f32x4_t G1 = zero4, G2 = zero4, G3 = zero4;   // Mka, Mbr, Mkr
 #pragma unroll
   for (int hf = 0; hf < 2; ++hf) {
-    if (staged) {
-      if (hf == 0) __builtin_amdgcn_s_setprio(1); else __builtin_amdgcn_s_setprio(2);
-    }
     // ---- v in fp16, row-major (the consumers read it transposed)
     {
       float fv[8];
@@ -316,7 +313,6 @@ __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags
       G3 = mfma(kA, qB, G3);        // Mkr[m][n] = kh_m . qt_n
     }
   }
-  if (staged) __builtin_amdgcn_s_setprio(3);
   // ---- triangular masks: earlier rows m for column n
   const int n = t;
   auto mask_tiles = [&](int i, bool lt, bool le, bool gt) {
@@ -372,7 +368,6 @@ __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags
     slot->keep_end = (lastseg == 0) ? 1 : 0;
     slot->keep_snap = (F.snap >= 0 && (!slow || seg_of(F.ns, F.snap) == 0)) ? 1 : 0;
   }
-  if (staged) __builtin_amdgcn_s_setprio(0);
 }
 
 // ---------------------------------------------------------------------------------------------------- consumer
@@ -381,7 +376,7 @@ __device__ __forceinline__ void produce(int lane, const Raw& x, const ChunkFlags
 // Byte offsets of this lane's operands inside a slot, computed once (the asm statement keeps the compiler from
 // recomputing them from the lane index in every chunk).
 struct LaneOffs {
-  uint32_t aq, l8, l16, vv, upd, gm;
+  uint32_t aq, l8, l16, vv, upd, gm, ypark;
 };
 __device__ __forceinline__ LaneOffs lane_offs(int q, int lane) {
   const int n = lane & 15, g = lane >> 4;
@@ -392,7 +387,8 @@ __device__ __forceinline__ LaneOffs lane_offs(int q, int lane) {
   o.vv = (uint32_t)(offsetof(Slot, V) + ((4 * g + (n >> 2)) * RS + 16 * q + 4 * (n & 3)) * 2);
   o.upd = (uint32_t)(offsetof(Slot, BK) + ((4 * g + (n >> 2)) * RS + 4 * (n & 3)) * 2);
   o.gm = (uint32_t)(offsetof(Slot, gamma) + 16 * g);
-  asm volatile("" : "+v"(o.aq), "+v"(o.l8), "+v"(o.l16), "+v"(o.vv), "+v"(o.upd), "+v"(o.gm));
+  o.ypark = (uint32_t)(offsetof(Slot, V) + ((4 * g) * RS + 16 * q + n) * 2);
+  asm volatile("" : "+v"(o.aq), "+v"(o.l8), "+v"(o.l16), "+v"(o.vv), "+v"(o.upd), "+v"(o.gm), "+v"(o.ypark));
   return o;
 }
 struct Consumer {
@@ -465,7 +461,7 @@ __device__ __forceinline__ void store_state_tile(void* p, int f32, size_t off, c
 
 // The state-dependent part of one chunk.  `next` is the slot of the chunk handled after this one (null after the
 // last one); `next_ready` waits until its producer has published it.  Returns false when that wait ran out.
-template <class PeekNext, class WaitNext>
+template <bool PARK, class PeekNext, class WaitNext>
 __device__ __forceinline__ bool consume(Consumer& C, Ops& o, const Slot* __restrict__ slot,
                                         const Slot* __restrict__ next, const SnapSlot* __restrict__ snapslot,
                                         const Wkv7Args& A, int64_t b, int64_t h, int nvalid, bool is_snap, bool q2drop,
@@ -545,12 +541,25 @@ __device__ __forceinline__ bool consume(Consumer& C, Ops& o, const Slot* __restr
   }
   // outputs: register i is token 4g+i, lanes n = 16 consecutive values
   const uint32_t y01 = pack_rn(Y[0], Y[1]), y23 = pack_rn(Y[2], Y[3]);
+  if (PARK) {
+    // The launch that also writes `sa`: y is parked in the value columns of V that only this wave reads (it fetched
+    // them a chunk ahead), and the producer that takes the slot next writes the chunk's y to memory as whole rows.
+    // Eight narrow stores per chunk hold the consumers up; four do not (measured: 4.5 % off this launch, while the
+    // launch without `sa` is 5 % slower this way and keeps its direct stores).
+    char* const yp = reinterpret_cast<char*>(const_cast<Slot*>(slot)) + C.off.ypark;
+    *reinterpret_cast<uint16_t*>(yp) = (uint16_t)(y01 & 0xffffu);
+    *reinterpret_cast<uint16_t*>(yp + RS * 2) = (uint16_t)(y01 >> 16);
+    *reinterpret_cast<uint16_t*>(yp + 2 * RS * 2) = (uint16_t)(y23 & 0xffffu);
+    *reinterpret_cast<uint16_t*>(yp + 3 * RS * 2) = (uint16_t)(y23 >> 16);
+  }
   char* const yl = oc.y + (size_t)oc.voff * 2;
   if (nvalid == CK) {
-    *reinterpret_cast<uint16_t*>(yl) = (uint16_t)(y01 & 0xffffu);
-    *reinterpret_cast<uint16_t*>(yl + oc.tok_bytes) = (uint16_t)(y01 >> 16);
-    *reinterpret_cast<uint16_t*>(yl + 2 * oc.tok_bytes) = (uint16_t)(y23 & 0xffffu);
-    *reinterpret_cast<uint16_t*>(yl + 3 * oc.tok_bytes) = (uint16_t)(y23 >> 16);
+    if (!PARK) {
+      *reinterpret_cast<uint16_t*>(yl) = (uint16_t)(y01 & 0xffffu);
+      *reinterpret_cast<uint16_t*>(yl + oc.tok_bytes) = (uint16_t)(y01 >> 16);
+      *reinterpret_cast<uint16_t*>(yl + 2 * oc.tok_bytes) = (uint16_t)(y23 & 0xffffu);
+      *reinterpret_cast<uint16_t*>(yl + 3 * oc.tok_bytes) = (uint16_t)(y23 >> 16);
+    }
     if (oc.sa != nullptr) {      // the residual for the backward pass, in fp16 like the operand it was used as
       char* const sl = oc.sa + (size_t)oc.voff * 2;
       *reinterpret_cast<uint16_t*>(sl) = (uint16_t)(sp[0] & 0xffffu);
@@ -564,7 +573,7 @@ __device__ __forceinline__ bool consume(Consumer& C, Ops& o, const Slot* __restr
     for (int i = 0; i < 4; ++i) {
       if (4 * g + i < nvalid) {
         const uint32_t yv = (i & 2) ? y23 : y01;
-        *reinterpret_cast<uint16_t*>(yl + i * oc.tok_bytes) = (uint16_t)((i & 1) ? (yv >> 16) : (yv & 0xffffu));
+        if (!PARK) *reinterpret_cast<uint16_t*>(yl + i * oc.tok_bytes) = (uint16_t)((i & 1) ? (yv >> 16) : (yv & 0xffffu));
         if (oc.sa != nullptr) {
           const uint32_t sv2 = sp[i >> 1];
           *reinterpret_cast<uint16_t*>(oc.sa + (size_t)oc.voff * 2 + i * oc.tok_bytes) =
@@ -578,11 +587,27 @@ __device__ __forceinline__ bool consume(Consumer& C, Ops& o, const Slot* __restr
   return ok;
 }
 
+// y of chunk jj, parked in the slot by the consumers, to memory: lane l stores 16 bytes of rows l/8 and l/8 + 8
+__device__ __forceinline__ void flush_y(const Slot* __restrict__ slot, const Wkv7Args& A, int64_t b, int64_t h, int jj,
+                                        int nch, int lane) {
+  const int nvalid = (jj + 1 < nch || A.T % CK == 0) ? CK : (int)(A.T % CK);
+  const int r = lane >> 3, piece = lane & 7;
+  char* const y0 = reinterpret_cast<char*>(A.out) +
+                   ((((size_t)b * A.T + (size_t)jj * CK + r) * A.H + h) * 64 + 8 * piece) * 2;
+  const uint4 lo = *reinterpret_cast<const uint4*>(&slot->V[r][8 * piece]);
+  const uint4 hi = *reinterpret_cast<const uint4*>(&slot->V[r + 8][8 * piece]);
+  if (r < nvalid) *reinterpret_cast<uint4*>(y0) = lo;
+  if (r + 8 < nvalid) *reinterpret_cast<uint4*>(y0 + (size_t)8 * A.H * 128) = hi;
+}
+
 }  // namespace
 
 // Step j handles chunk j in slot j % RING.  Producer p fills the slot once every consumer has released step j - RING,
 // then publishes ready = j + 1; consumers take the steps in order.  Every wait is for a strictly earlier step, so
 // the hand-shake cannot cycle.
+// PARK: the consumers leave y in the slot and the producers write it out (see `consume`); steps nch .. nch + RING - 1
+// of the producers then produce nothing and only write out the y of the last RING chunks.
+template <bool PARK>
 __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_fwd_kernel(Wkv7Args A) {
   extern __shared__ __align__(16) unsigned char smem_raw[];
   Slot* slots = reinterpret_cast<Slot*>(smem_raw);
@@ -641,7 +666,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_fwd_kernel(Wkv7Args
       const int nvalid = (j + 1 < nch || A.T % CK == 0) ? CK : (int)(A.T % CK);
       const int sn = (si + 1 == RING) ? 0 : si + 1;
       const Slot* next = (j + 1 < nch) ? &slots[sn] : nullptr;
-      ok = consume(C, ops, &slots[si], next, snapslot, A, b, h, nvalid, j == csnap, q2drop, oc,
+      ok = consume<PARK>(C, ops, &slots[si], next, snapslot, A, b, h, nvalid, j == csnap, q2drop, oc,
                    [&]() { return peek_ready(sy, sn); },
                    [&](int peeked) {
                      return wait_ready_peeked(sy, sn, j + 2, peeked);
@@ -662,14 +687,23 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_fwd_kernel(Wkv7Args
       load_raw(raw, A, b, h, (int64_t)p * CK, lane);
       ns_mine = chunk_flag_prefetch(A.ns, A.T, b, (int64_t)p * CK, lane);
     }
-    for (int j = p; j < nch; j += NPROD) {
+    for (int j = p; j < nch + (PARK ? RING : 0); j += NPROD) {
       const int64_t c0 = (int64_t)j * CK;
-      const ChunkFlags F = chunk_flags_of(A.ns, ns_mine, A.flags, A.T, c0, L);
       const int si = j % RING;
       Slot* slot = &slots[si];
-      if (j >= RING && !wait_consumed_lazy(sy, si, j - RING + 1, lane)) break;
+      if (PARK) {
+        // Retire the operand loads requested a step ago before anything else: loads and stores share the memory
+        // counter, and a wait for a load inside `produce` would otherwise also wait for the y stores issued below.
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
+      }
+      if (j >= RING) {
+        if (!wait_consumed_lazy(sy, si, j - RING + 1, lane)) break;
+        if (PARK) flush_y(slot, A, b, h, j - RING, nch, lane);
+      }
+      if (PARK && j >= nch) continue;
+      const ChunkFlags F = chunk_flags_of(A.ns, ns_mine, A.flags, A.T, c0, L);
       mask_raw(raw, F.nvalid, lane);
-      produce(lane, raw, F, slot, snapslot, events_word(A.status), A.sa == nullptr);
+      produce(lane, raw, F, slot, snapslot, events_word(A.status));
       if (j + NPROD < nch) {
         load_raw(raw, A, b, h, c0 + (int64_t)NPROD * CK, lane);
         ns_mine = chunk_flag_prefetch(A.ns, A.T, b, c0 + (int64_t)NPROD * CK, lane);
@@ -691,10 +725,18 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_fwd_kernel(Wkv7Args
 hipError_t launch_wkv7_chunk_fwd(const Wkv7Args& A, hipStream_t stream) {
   static_assert(RING <= MAX_RING, "the hand-shake words cover MAX_RING slots");
   const size_t smem = RING * sizeof(Slot) + sizeof(SnapSlot) + sizeof(Sync);
-  static LdsAttrOnce once;
-  const hipError_t attr = allow_dynamic_lds(once, reinterpret_cast<const void*>(wkv7_fwd_kernel), smem);
-  if (attr != hipSuccess) return attr;
-  hipLaunchKernelGGL(wkv7_fwd_kernel, dim3((unsigned)(A.B * A.H)), dim3(64 * (NCONS + NPROD)), smem, stream, A);
+  const dim3 grid((unsigned)(A.B * A.H)), block(64 * (NCONS + NPROD));
+  if (A.sa != nullptr) {
+    static LdsAttrOnce once;
+    const hipError_t attr = allow_dynamic_lds(once, reinterpret_cast<const void*>(wkv7_fwd_kernel<true>), smem);
+    if (attr != hipSuccess) return attr;
+    hipLaunchKernelGGL(wkv7_fwd_kernel<true>, grid, block, smem, stream, A);
+  } else {
+    static LdsAttrOnce once;
+    const hipError_t attr = allow_dynamic_lds(once, reinterpret_cast<const void*>(wkv7_fwd_kernel<false>), smem);
+    if (attr != hipSuccess) return attr;
+    hipLaunchKernelGGL(wkv7_fwd_kernel<false>, grid, block, smem, stream, A);
+  }
   return hipGetLastError();
 }
 
