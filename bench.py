@@ -29,9 +29,9 @@ B, T, H, N = 8, 4096, 32, 64
 # figures in profiles/), each with the sha1 prefix of the kernel source it was measured on: when the source has
 # changed since, `roofline.traffic` is null instead of a stale figure.
 MEASURED_TRAFFIC = {
-    "wkv7_fwd": (948.5e6, "wkv7_fwd.hip", "8b8165f4cd20", "profiles/wkv7_fwd_B8_T4096_H32_bf16.md"),
+    "wkv7_fwd": (948.7e6, "wkv7_fwd.hip", "51a3d3ca403c", "profiles/wkv7_fwd_B8_T4096_H32_bf16.md"),
     "wkv4_fwd": (4028.7e6, "wkv4.hip", "d83a0992a92e", "profiles/wkv4_fwd_B32_T4096_C2560_f32.md"),
-    "wkv6_fwd": (688.4e6, "wkv6_fwd.hip", "0188be317e1c", "profiles/wkv6_fwd_bwd_B16_T2048_H32_bf16.md"),
+    "wkv6_fwd": (688.4e6, "wkv6_fwd.hip", "e577f9812ac6", "profiles/wkv6_fwd_bwd_B16_T2048_H32_bf16.md"),
 }
 
 
