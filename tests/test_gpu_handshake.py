@@ -51,6 +51,26 @@ def test_wkv7_forward_and_backward_poison_their_outputs_and_count():
     assert all(bool(torch.isfinite(g.float()).all()) for g in g2)
 
 
+def test_wkv7_forward_without_the_residual_poisons_its_outputs_and_counts():
+    """The launch without `sa` is an instantiation of its own (its consumers store y themselves; with `sa` the
+    producers write it out): the same failure path, checked separately."""
+    from jaxrwkv_amd import _lib, ops
+    args, _, _ = inputs7(seed=1)
+    good = ops.wkv7_fwd(*args, want_sa=False)
+    before = ops.handshake_failures()
+    new_s, y, sa = ops.wkv7_fwd(*args, want_sa=False, debug_flags=_lib.DEBUG_DROP_PUBLISH)
+    assert sa is None
+    assert ops.handshake_failures() - before == B * H
+    assert all_nan(new_s) and all_nan(y)
+    before = ops.handshake_failures()
+    again = ops.wkv7_fwd(*args, want_sa=False)
+    assert ops.handshake_failures() == before
+    assert torch.equal(again[0], good[0]) and torch.equal(again[1], good[1])
+    # both instantiations give the same y and state
+    with_sa = ops.wkv7_fwd(*args, want_sa=True)
+    assert torch.equal(with_sa[0], good[0]) and torch.equal(with_sa[1], good[1])
+
+
 def test_wkv6_forward_and_backward_poison_their_outputs_and_count():
     from jaxrwkv_amd import _lib, ops
     g = torch.Generator("cuda").manual_seed(1)

@@ -84,6 +84,22 @@ def test_bf16_state_dtype_and_no_sa():
     assert_close("new_s", new_s, ref_s, rtol=2.0 ** -7, atol=S_ATOL, scale_atol=True)
 
 
+@pytest.mark.parametrize("B,T,H,seed,p", [(1, 16, 1, 50, 0.0), (2, 17, 2, 51, 0.1), (1, 159, 2, 52, 0.05),
+                                          (2, 160, 1, 53, 0.0), (1, 161, 3, 54, 0.02), (2, 333, 2, 55, 0.01),
+                                          (1, 9, 1, 56, 0.2), (1, 1000, 2, 57, 0.004)])
+def test_the_two_instantiations_agree_bit_for_bit(B, T, H, seed, p):
+    """The launch without `sa` (consumers store y) and the one with it (y parked in LDS, written out by the producers,
+    the last slots by extra steps after the last chunk) must give the same bits; the first is also held to the oracle
+    here, the second by every other test of this file."""
+    x = wkv7_inputs(B, T, H, 64, seed=seed, bf16=True, p_reset=p, min_len_frac=0.3)
+    for compat in (True, False):
+        s0, y0, none = run(x, compat, want_sa=False)
+        s1, y1, sa1 = run(x, compat, want_sa=True)
+        assert none is None
+        assert np.array_equal(y0, y1) and np.array_equal(s0, s1)
+        check(x, compat, s0, y0, None)
+
+
 def test_matches_sequential_kernel_and_tvd_bar():
     x = wkv7_inputs(2, 1024, 4, 64, seed=41, bf16=True, p_reset=1.0 / 256)
     new_s, y, sa = run(x, True)
