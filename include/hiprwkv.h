@@ -139,7 +139,9 @@ size_t hiprwkv_wkv7_bwd_workspace_bytes(int64_t B, int64_t T, int64_t H, int64_t
  * Unlike the reference's native op it honours new_starts, takes the cotangent of the
  * returned state (gs_out, may be NULL = 0) and returns the one of the input state.
  * Three sweeps over the sequence on the matrix cores: bf16 hi+lo operand pairs beside bf16
- * I/O, fp32 operands (no rounding below fp32) beside fp32 I/O; HIPRWKV_FORCE_SEQ runs the
+ * I/O (the cotangent of `sa` passes between them as 16-bit fixed point with a power-of-two
+ * scale per 16 x 16 tile: 16 bits whatever the size of the cotangents), fp32 operands and an
+ * fp32 workspace (no rounding below fp32) beside fp32 I/O; HIPRWKV_FORCE_SEQ runs the
  * sequential fp32 sweeps instead. */
 int hiprwkv_wkv7_bwd(hiprwkv_stream stream, int io_dtype, int state_dtype,
                      int64_t B, int64_t T, int64_t H, int64_t N,

@@ -311,6 +311,52 @@ __device__ __forceinline__ size_t f_record(int64_t b, int64_t h, int64_t H, int 
   return ((((size_t)b * H + h) * nch + c) * NCONS + q) * F_REC;
 }
 
+// The WKV7 backward's workspace dsa (cotangent of sa, one value per token and value index) between the chunked bf16
+// sweeps: 16-bit signed fixed point with one power-of-two scale per (sequence, head, chunk, consumer wave of the
+// reverse sweep A = 16 tokens x 16 value indices), the scale exponents kept as int32 in a side array.  A tile is scaled
+// by 2^k so that its largest magnitude lands in [1/2, 1) and rounded to multiples of 1/32767: an absolute error of at
+// most 1.6e-5 of the tile's largest magnitude, against 2^-17 relative for the bf16 pairs the sweeps make of it and
+// 2^-12 relative for an IEEE half (which put single elements of ga at twice the tolerance of the tests).  Every use of
+// dsa is a sum over the value index, so an error that is absolute within a tile is the right kind.  A tile that holds
+// inf or NaN gets the exponent DSA_BAD, which makes every value of it NaN for the reader.
+constexpr int DSA_BAD = 0x7fffffff;
+__device__ __forceinline__ int* dsa_scales(float* side, int64_t b, int64_t h, int64_t H, int nch, int c) {
+  return reinterpret_cast<int*>(side) + (((size_t)b * H + h) * nch + c) * NCONS;
+}
+template <int CTRL>
+__device__ __forceinline__ float dpp_max(float x) {
+  return fmaxf(x, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true)));
+}
+// x: this lane's four accumulator registers of the tile (any layout); the result is uniform over the wave
+__device__ __forceinline__ int dsa_scale_exponent(const f32x4_t x) {
+  float m = fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3])));
+  m = dpp_max<0x111>(m);      // row_shr:1, 2, 4, 8: lane 15 of every row of 16 holds the row's maximum
+  m = dpp_max<0x112>(m);
+  m = dpp_max<0x114>(m);
+  m = dpp_max<0x118>(m);
+  auto row_max = [&](int l) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(m), l)); };
+  const float mw = fmaxf(fmaxf(row_max(15), row_max(31)), fmaxf(row_max(47), row_max(63)));
+  const int e = (__float_as_int(mw) >> 23) & 0xff;      // biased exponent of the largest magnitude
+  const float sum = (x[0] + x[1]) + (x[2] + x[3]);      // NaN if any element is (the maximum skips NaNs)
+  const bool bad = __ballot(sum != sum) != 0ull || e == 255;
+  return bad ? DSA_BAD : 126 - e;                       // largest magnitude * 2^k in [1/2, 1)
+}
+// two values of a tile to fixed point (v_cvt_pknorm_i16_f32: round(x * 32767), clamped)
+__device__ __forceinline__ uint32_t pack_dsa2(float x0, float x1, int kexp) {
+  typedef short s2_t __attribute__((ext_vector_type(2)));
+  const int k = kexp == DSA_BAD ? 0 : kexp;
+  const s2_t p = __builtin_amdgcn_cvt_pknorm_i16(__builtin_amdgcn_ldexpf(x0, k), __builtin_amdgcn_ldexpf(x1, k));
+  return __builtin_bit_cast(uint32_t, p);
+}
+// eight such values of one lane back to fp32
+__device__ __forceinline__ void unpack_dsa8(const uint4 raw, int kexp, float4& lo4, float4& hi4) {
+  const float mult = kexp == DSA_BAD ? __int_as_float(0x7fc00000) : __builtin_amdgcn_ldexpf(1.0f / 32767.0f, -kexp);
+  auto lo = [&](uint32_t w) { return (float)((int)(w << 16) >> 16) * mult; };
+  auto hi = [&](uint32_t w) { return (float)((int)w >> 16) * mult; };
+  lo4 = make_float4(lo(raw.x), hi(raw.x), lo(raw.y), hi(raw.y));
+  hi4 = make_float4(lo(raw.z), hi(raw.z), lo(raw.w), hi(raw.w));
+}
+
 // Selection operands that turn an MFMA into a transposer: against an A operand whose k-slot (g, jj) stands for key
 // 8g + jj of a 32-key half, B = sel[x] yields D[token][n] = value at key 16x + n.
 __device__ __forceinline__ void make_sel(u32x4_t (&sel)[2], int lane) {

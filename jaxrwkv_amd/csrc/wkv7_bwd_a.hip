@@ -389,8 +389,9 @@ __device__ __forceinline__ void load_ops(Ops& o, const Slot* __restrict__ slot, 
 // Uniform output cursors of a consumer, moved by one chunk per call.
 struct OutCursor {
   char* y;             // A.gv at (b, c0, h, 0)
-  char* sa;            // A.dsa at the same place
-  size_t tok_bytes;    // bytes between consecutive tokens in y (twice that in sa)
+  char* sa;            // A.dsa at the same place (16-bit fixed point scaled per chunk and wave: chunk_common.h)
+  int* scale;          // this wave's scale exponent of the chunk
+  size_t tok_bytes;    // bytes between consecutive tokens in y and in sa
   uint32_t voff;       // lane part of the address, in elements: (4g * H) * 64 + value
 };
 
@@ -529,28 +530,34 @@ __device__ __forceinline__ bool consume(Consumer& C, Ops& o, const Slot* __restr
   // outputs: register i is token 4g+i, lanes n = 16 consecutive values
   const uint32_t y01 = pack_rn(Y[0], Y[1]), y23 = pack_rn(Y[2], Y[3]);
   char* const yl = oc.y + (size_t)oc.voff * 2;
+  // dsa leaves as 16-bit fixed point with one power-of-two scale per chunk and wave (chunk_common.h), at half the
+  // bytes of fp32; the exponent goes to a side array.
+  const int kexp = dsa_scale_exponent(SA);
+  const uint32_t d01 = pack_dsa2(SA[0], SA[1], kexp), d23 = pack_dsa2(SA[2], SA[3], kexp);
+  if (lane == 0) *oc.scale = kexp;
+  char* const sl = oc.sa + (size_t)oc.voff * 2;
   if (nvalid == CK) {
     *reinterpret_cast<uint16_t*>(yl) = (uint16_t)(y01 & 0xffffu);
     *reinterpret_cast<uint16_t*>(yl + oc.tok_bytes) = (uint16_t)(y01 >> 16);
     *reinterpret_cast<uint16_t*>(yl + 2 * oc.tok_bytes) = (uint16_t)(y23 & 0xffffu);
     *reinterpret_cast<uint16_t*>(yl + 3 * oc.tok_bytes) = (uint16_t)(y23 >> 16);
-    if (oc.sa != nullptr) {
-      char* const sl = oc.sa + (size_t)oc.voff * 4;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) *reinterpret_cast<float*>(sl + 2 * i * oc.tok_bytes) = SA[i];
-    }
+    *reinterpret_cast<uint16_t*>(sl) = (uint16_t)(d01 & 0xffffu);
+    *reinterpret_cast<uint16_t*>(sl + oc.tok_bytes) = (uint16_t)(d01 >> 16);
+    *reinterpret_cast<uint16_t*>(sl + 2 * oc.tok_bytes) = (uint16_t)(d23 & 0xffffu);
+    *reinterpret_cast<uint16_t*>(sl + 3 * oc.tok_bytes) = (uint16_t)(d23 >> 16);
   } else {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       if (4 * g + i < nvalid) {
-        const uint32_t yv = (i & 2) ? y23 : y01;
+        const uint32_t yv = (i & 2) ? y23 : y01, dv = (i & 2) ? d23 : d01;
         *reinterpret_cast<uint16_t*>(yl + i * oc.tok_bytes) = (uint16_t)((i & 1) ? (yv >> 16) : (yv & 0xffffu));
-        if (oc.sa != nullptr) *reinterpret_cast<float*>(oc.sa + (size_t)oc.voff * 4 + 2 * i * oc.tok_bytes) = SA[i];
+        *reinterpret_cast<uint16_t*>(sl + i * oc.tok_bytes) = (uint16_t)((i & 1) ? (dv >> 16) : (dv & 0xffffu));
       }
     }
   }
   oc.y -= CK * oc.tok_bytes;
-  oc.sa -= 2 * CK * oc.tok_bytes;
+  oc.sa -= CK * oc.tok_bytes;
+  oc.scale -= 4;
 
   return ok;
 }
@@ -594,7 +601,8 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_bwd_a_kernel(Wkv7Ar
     oc.tok_bytes = (size_t)A.H * 64 * 2;
     const size_t el0 = (((size_t)b * A.T + first_tok) * A.H + h) * 64;
     oc.y = reinterpret_cast<char*>(A.gv) + el0 * 2;
-    oc.sa = reinterpret_cast<char*>(A.dsa) + el0 * 4;
+    oc.sa = reinterpret_cast<char*>(A.dsa) + el0 * 2;
+    oc.scale = dsa_scales(A.e3, b, h, A.H, nch, nch - 1) + wave;
 
     oc.voff = (uint32_t)((4 * (lane >> 4)) * (int)A.H * 64 + 16 * wave + (lane & 15));
     const int csnap = (L >= 1 && inject) ? (int)((L - 1) / CK) : -1;
@@ -657,7 +665,7 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_bwd_a_kernel(Wkv7Ar
   __syncthreads();
   if (head_broken(sy, A.status)) {
     poison_token_rows(A.gv, 2, b, h, A.T, A.H);
-    poison_token_rows(A.dsa, 4, b, h, A.T, A.H);
+    poison_token_rows(A.dsa, 2, b, h, A.T, A.H);
     poison_state(A.gs, A.st_f32, b, h, A.H);
   }
 }

@@ -75,7 +75,8 @@ struct __attribute__((aligned(16))) SnapSlot {
 struct Raw {
   uint4 w[2], r[2], a[2], v[2], dy[2];
   uint4 sa[2];             // the forward residual, fp16
-  float4 dsa[2][2];
+  uint4 dsa[2];            // sweep A's workspace: 16-bit fixed point, scaled per chunk and value tile (chunk_common.h)
+  int4 dsk;                // k of the chunk's four value tiles
   uint4 k[2], b[2];        // passed on to the consumers as they are
   float4 f[NCONS];         // lane l: entry l of each consumer wave's record of this chunk
 };
@@ -88,27 +89,21 @@ __device__ __forceinline__ void load_raw(Raw& x, const Wkv7Args& A, int64_t b, i
 #pragma unroll
     for (int q = 0; q < NCONS; ++q) x.f[q] = rec[64 * q + lane];
   }
+  x.dsk = *reinterpret_cast<const int4*>(dsa_scales(A.e3, b, h, A.H, (int)((A.T + CK - 1) / CK), (int)(c0 / CK)));
   if (c0 + t < A.T) {
     const size_t el = (((size_t)b * A.T + c0 + t) * A.H + h) * 64 + 8 * g;
     auto ld = [&](const void* p, uint4 (&o)[2]) {
       o[0] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(p) + el * 2);
       o[1] = *reinterpret_cast<const uint4*>(reinterpret_cast<const char*>(p) + el * 2 + 64);
     };
-    auto ld32 = [&](const float* p, float4 (&o)[2][2]) {
-      o[0][0] = *reinterpret_cast<const float4*>(p + el);
-      o[0][1] = *reinterpret_cast<const float4*>(p + el + 4);
-      o[1][0] = *reinterpret_cast<const float4*>(p + el + 32);
-      o[1][1] = *reinterpret_cast<const float4*>(p + el + 36);
-    };
     ld(A.w, x.w); ld(A.r, x.r); ld(A.a, x.a); ld(A.v, x.v); ld(A.gy, x.dy);
-    ld(A.sa_in, x.sa); ld32(A.dsa, x.dsa);
+    ld(A.sa_in, x.sa); ld(A.dsa, x.dsa);
     ld(A.k, x.k); ld(A.b, x.b);
   } else {
     const uint4 z = make_uint4(0, 0, 0, 0);
-    const float4 zf = make_float4(0.f, 0.f, 0.f, 0.f);
     x.w[0] = x.w[1] = x.r[0] = x.r[1] = x.a[0] = x.a[1] = x.v[0] = x.v[1] = x.dy[0] = x.dy[1] = z;
     x.sa[0] = x.sa[1] = x.k[0] = x.k[1] = x.b[0] = x.b[1] = z;
-    x.dsa[0][0] = x.dsa[0][1] = x.dsa[1][0] = x.dsa[1][1] = zf;
+    x.dsa[0] = x.dsa[1] = z;
   }
 }
 
@@ -266,7 +261,12 @@ __device__ __forceinline__ void produce(const Producer& P, const Raw& x, const C
       const u32x4_t dyop = {dr.x, dr.y, dr.z, dr.w};
       u32x4_t sa_h, sa_l, ds_h, ds_l;
       split8h(x.sa[hf], sa_h, sa_l);
-      split8(x.dsa[hf][0], x.dsa[hf][1], ds_h, ds_l);
+      {
+        float4 d_lo, d_hi;
+        const int kq = hf == 0 ? ((g >> 1) ? x.dsk.y : x.dsk.x) : ((g >> 1) ? x.dsk.w : x.dsk.z);
+        unpack_dsa8(x.dsa[hf], kq, d_lo, d_hi);
+        split8(d_lo, d_hi, ds_h, ds_l);
+      }
       put(slot->V[t], vop, row_keep);
       put(slot->SA[0][t], sa_h, row_keep);
       put(slot->SA[1][t], sa_l, row_keep);

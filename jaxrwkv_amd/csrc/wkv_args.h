@@ -22,7 +22,11 @@ struct Wkv7Args {
   const void* sa_in;     // the forward residual, in the forward's type
   const void* gs_out;
   void *gw, *gr, *gk, *gv, *ga, *gb, *gs;
-  float *dsa, *e2, *e3;  // workspace, (B,T,H,64) fp32 each (the chunked sweeps keep e3_t + e2_{t+1} in e2, as records per chunk and wave: chunk_common.h f_record; e3 unused)
+  // workspace, three regions of (B,T,H,64) fp32 each.  The sequential sweeps and the chunked fp32 ones keep dsa in the
+  // first as fp32; the chunked bf16 sweeps keep it there as 16-bit fixed point with one scale exponent per chunk and
+  // value tile, the exponents in the third region (chunk_common.h dsa_scales).  The chunked sweeps keep e3_t + e2_{t+1}
+  // in e2, as records per chunk and wave (chunk_common.h f_record), and do not use e3 otherwise.
+  float *dsa, *e2, *e3;
   unsigned* status;      // device word counting workgroups whose hand-shake gave up (may be null)
   // Elements between the states of consecutive sequences in `s` / `new_s`; 0 = dense (H*64*64).  Honoured by the
   // small-T kernel only (states read and written inside a packed model state).

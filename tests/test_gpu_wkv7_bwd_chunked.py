@@ -91,3 +91,33 @@ def test_matches_sequential_sweeps():
     check(seq, ref)
     for n in NAMES:
         assert_close("chunked-vs-sequential g" + n, got[n], seq[n], rtol=RTOL[n], atol=ATOL[n], scale_atol=True)
+
+
+@pytest.mark.parametrize("shift", [-40, -17, 12, 30])
+def test_cotangents_scale_by_powers_of_two_exactly(shift):
+    """The workspace between the sweeps is 16-bit fixed point with a power-of-two scale per 16 x 16 tile, chosen from
+    the tile's largest magnitude; every other step is fp32 arithmetic or a bf16 pair.  Multiplying dy and the state
+    cotangent by 2^shift must therefore multiply every cotangent by 2^shift to the bit (as long as nothing leaves the
+    normal range): gradients 1e-12 or 1e9 times the usual size keep their 16 bits."""
+    x = wkv7_inputs(2, 150, 2, 64, seed=61, bf16=True, p_reset=0.03, min_len_frac=0.4)
+    base = run(x, True)
+    c = 2.0 ** shift
+    y = dict(x)
+    y["dy"], y["ds"] = x["dy"] * c, x["ds"] * c
+    scaled = run(y, True)
+    for n in NAMES:
+        assert np.array_equal(scaled[n], base[n] * c), n
+
+
+def test_a_non_finite_cotangent_stays_visible():
+    """A tile of the workspace that holds inf or NaN is marked as a whole, so the sweeps that read it cannot turn a
+    non-finite value into a finite one."""
+    x = wkv7_inputs(1, 64, 1, 64, seed=62, bf16=True, resets=False)
+    x["length"][:] = 64
+    for bad in (np.inf, np.nan):
+        y = dict(x)
+        y["dy"] = x["dy"].copy()
+        y["dy"][0, 37, 0, 5] = bad
+        g = run(y, True)
+        for n in ("r", "k", "a", "b", "w"):
+            assert not np.all(np.isfinite(g[n][0, :38])), (bad, n)
