@@ -323,23 +323,27 @@ constexpr int DSA_BAD = 0x7fffffff;
 __device__ __forceinline__ int* dsa_scales(float* side, int64_t b, int64_t h, int64_t H, int nch, int c) {
   return reinterpret_cast<int*>(side) + (((size_t)b * H + h) * nch + c) * NCONS;
 }
-template <int CTRL>
-__device__ __forceinline__ float dpp_max(float x) {
-  return fmaxf(x, __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true)));
+// x: this lane's four accumulator registers of the tile (any layout); the result is uniform over the wave.  The
+// maximum runs over the magnitudes' bit patterns as unsigned integers, which orders finite < inf < NaN, so one biased
+// exponent of 255 at the end stands for "inf or NaN somewhere in the tile".
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ uint32_t dpp_umax(uint32_t x) {
+  const uint32_t y = (uint32_t)__builtin_amdgcn_update_dpp((int)x, (int)x, CTRL, ROW_MASK, 0xf, false);
+  return x > y ? x : y;
 }
-// x: this lane's four accumulator registers of the tile (any layout); the result is uniform over the wave
 __device__ __forceinline__ int dsa_scale_exponent(const f32x4_t x) {
-  float m = fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3])));
-  m = dpp_max<0x111>(m);      // row_shr:1, 2, 4, 8: lane 15 of every row of 16 holds the row's maximum
-  m = dpp_max<0x112>(m);
-  m = dpp_max<0x114>(m);
-  m = dpp_max<0x118>(m);
-  auto row_max = [&](int l) { return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(m), l)); };
-  const float mw = fmaxf(fmaxf(row_max(15), row_max(31)), fmaxf(row_max(47), row_max(63)));
-  const int e = (__float_as_int(mw) >> 23) & 0xff;      // biased exponent of the largest magnitude
-  const float sum = (x[0] + x[1]) + (x[2] + x[3]);      // NaN if any element is (the maximum skips NaNs)
-  const bool bad = __ballot(sum != sum) != 0ull || e == 255;
-  return bad ? DSA_BAD : 126 - e;                       // largest magnitude * 2^k in [1/2, 1)
+  auto mag = [](float v) { return (uint32_t)__float_as_int(v) & 0x7fffffffu; };
+  const uint32_t m01 = mag(x[0]) > mag(x[1]) ? mag(x[0]) : mag(x[1]);
+  const uint32_t m23 = mag(x[2]) > mag(x[3]) ? mag(x[2]) : mag(x[3]);
+  uint32_t m = m01 > m23 ? m01 : m23;
+  m = dpp_umax<0x111, 0xf>(m);      // row_shr:1, 2, 4, 8: lane 15 of every row of 16 holds the row's maximum
+  m = dpp_umax<0x112, 0xf>(m);
+  m = dpp_umax<0x114, 0xf>(m);
+  m = dpp_umax<0x118, 0xf>(m);
+  m = dpp_umax<0x142, 0xa>(m);      // row_bcast:15 into rows 1 and 3: lanes 31 and 63 hold the maxima of their row pairs
+  m = dpp_umax<0x143, 0xc>(m);      // row_bcast:31 into rows 2 and 3: lane 63 holds the wave's maximum
+  const int e = (int)((uint32_t)__builtin_amdgcn_readlane((int)m, 63) >> 23);      // biased exponent of it
+  return e == 255 ? DSA_BAD : 126 - e;                  // largest magnitude * 2^k in [1/2, 1)
 }
 // two values of a tile to fixed point (v_cvt_pknorm_i16_f32: round(x * 32767), clamped)
 __device__ __forceinline__ uint32_t pack_dsa2(float x0, float x1, int kexp) {
