@@ -268,7 +268,7 @@ def bench_wkv7(torch, ops, args):
                           "hbm_frac": fb_bytes / (ms2 * 1e-3) / 1e9 / HBM_PEAK_GBS, "algorithmic_bytes": fb_bytes,
                           "note": "forward keeps the residual sa (fp16 beside bf16 I/O); backward = three sweeps (reverse, forward, reverse), " +
                                   ("sequential fp32 VALU kernels" if args.seq else "chunked MFMA kernels") +
-                                  "; dsa and the decay-gradient terms pass through an fp32 workspace"}
+                                  "; dsa passes between them as 16-bit fixed point with a scale per 16x16 tile, the decay-gradient terms as fp32 records"}
         if not args.no_power:
             out["fwd_bwd"]["power"] = power_probe(torch, fwd_bwd)
     if not args.no_fp32:
