@@ -665,7 +665,8 @@ __global__ __launch_bounds__(64 * (NCONS + NPROD)) void wkv7_bwd_a_kernel(Wkv7Ar
   __syncthreads();
   if (head_broken(sy, A.status)) {
     poison_token_rows(A.gv, 2, b, h, A.T, A.H);
-    poison_token_rows(A.dsa, 2, b, h, A.T, A.H);
+    // the workspace of this (sequence, head) reads as NaN for the next two sweeps: every tile gets the reserved exponent
+    for (int i = threadIdx.x; i < nch * NCONS; i += blockDim.x) dsa_scales(A.e3, b, h, A.H, nch, 0)[i] = DSA_BAD;
     poison_state(A.gs, A.st_f32, b, h, A.H);
   }
 }
